@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the flash-decode hot path on one MI355X.
+
+A "step" is one decode call (split-KV kernel + LSE combine) over one batch of synthetic, HBM-resident
+inputs.  Default workload: the Llama-3-8B decode shape (batch 32, 32 q heads / 8 kv heads, head_dim 128,
+kv_len 4096, page size 16, bf16).  Prints ONE JSON line:
+
+  value          achieved HBM GB/s of the whole call = algorithmic bytes / measured time per call
+  us_per_call    the same measurement as a latency
+  roofline       the split-KV kernel alone against the 8 TB/s HBM peak, its launches timed with HIP
+                 events on the launch stream
+  cpu_baseline   the torch restatement of the reference's torch implementation on this box's host cores,
+                 timed on a bounded sample of the same inputs (a baseline, not the target)
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME] [--rotate R] [--kv-split S]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--config", default="llama3_8b_b32")
+    ap.add_argument("--rotate", type=int, default=2,
+                    help="distinct KV pools cycled through, so the working set exceeds the 256 MB memory-side cache")
+    ap.add_argument("--kv-split", type=int, default=-1)
+    ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def cpu_baseline(inp, budget_s: float):
+    """Time oracle.paged_attn.ref_paged_attn on the host cores for a sample of sequences."""
+    import torch
+    from oracle.paged_attn import ref_paged_attn
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    lens = inp.kv_lens_host
+    batch = len(lens)
+
+    def run(rows):
+        t0 = time.perf_counter()
+        ref_paged_attn(inp.q[rows], inp.k_cache, inp.v_cache, [lens[i] for i in rows], inp.block_table[rows],
+                       inp.sm_scale)
+        return time.perf_counter() - t0
+
+    # fp8 cache: the reference behaviour is "dequantise to bf16, then the same decode"; the sample pays
+    # for the dequantisation of its own pages only.
+    if inp.cfg.kv_dtype == "fp8_e4m3":
+        from oracle.fp8 import dequant_per_head
+
+        def run(rows):  # noqa: F811
+            t0 = time.perf_counter()
+            for i in rows:
+                n_pg = (lens[i] + inp.cfg.page_size - 1) // inp.cfg.page_size
+                ids = inp.block_table[i, :n_pg].long()
+                kd = dequant_per_head(inp.k_cache[ids], inp.k_scale)
+                vd = dequant_per_head(inp.v_cache[ids], inp.v_scale)
+                tbl = torch.arange(n_pg, dtype=torch.int32)[None]
+                ref_paged_attn(inp.q[i:i + 1], kd, vd, [lens[i]], tbl, inp.sm_scale)
+            return time.perf_counter() - t0
+
+    run([0])                                   # warm-up
+    t_one = run([0])
+    n_rows = max(1, min(batch, int(budget_s / 3 / max(t_one, 1e-4))))
+    rows = list(range(n_rows))
+    best = min(run(rows) for _ in range(3))
+    tokens_sample = sum(lens[i] for i in rows)
+    tokens_all = sum(lens)
+    est_call_s = best * tokens_all / max(tokens_sample, 1)
+    return {
+        "value": inp.algorithmic_bytes() / est_call_s / 1e9,
+        "unit": "GB/s",
+        "us_per_call": est_call_s * 1e6,
+        "cores": cores,
+        "kind": "port",
+        "sample": (f"oracle ref_paged_attn (torch CPU, bf16) on sequences 0..{n_rows - 1} of {batch}, best of 3, "
+                   f"scaled by attended tokens ({tokens_sample}/{tokens_all})" +
+                   ("" if n_rows < batch else "; full batch")),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's share of the decode path; --gpus {args.gpus} is not supported "
+              "(this build has no multi-GPU leg)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path for the kernels)", file=sys.stderr)
+        sys.exit(2)
+    import triton_distributed_amd as tda
+    from triton_distributed_amd import workloads as wl
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    t_gen = time.perf_counter()
+    inp_cpu = wl.make_inputs(args.config)
+    print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
+    inp = inp_cpu.to(dev)
+    pools = [(inp.k_cache, inp.v_cache)]
+    for r in range(1, max(1, args.rotate)):
+        # further pools: same pages, different (seeded) contents - the access pattern is identical
+        g = torch.Generator(device=dev).manual_seed(inp.cfg.seed + 100 * r)
+        if inp.cfg.kv_dtype == "fp8_e4m3":
+            mk = lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
+                torch.float8_e4m3fn)
+        else:
+            mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=torch.bfloat16)
+        pools.append((mk(), mk()))
+    calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
+                                v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
+                                max_kv_len=max(inp.kv_lens_host))
+             for k, v in pools]
+    plan = calls[0].plan
+    alg_bytes = inp.algorithmic_bytes()
+
+    # sanity of the timed configuration (parity proper is the job of tests/ and __graft_entry__.smoke())
+    out, lse = calls[0].run()
+    torch.cuda.synchronize()
+    if not (torch.isfinite(out.float()).all() and torch.isfinite(lse).all()):
+        raise RuntimeError("non-finite decode output on the benchmark inputs")
+
+    def step(i):
+        calls[i % len(calls)].run()
+
+    # ---- whole call: W warm-up, then exactly K timed steps ----------------------------------------------------
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms_per_step = wall_s * 1e3 / args.steps
+    gbps = alg_bytes / (wall_s / args.steps) / 1e9
+
+    # ---- dominant kernel alone (split-KV), HIP events on the launch stream ------------------------------------
+    for i in range(min(args.warmup, 10)):
+        calls[i % len(calls)].run_splitkv()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(args.steps):
+        calls[i % len(calls)].run_splitkv()
+    e1.record()
+    torch.cuda.synchronize()
+    split_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    split_gbps = alg_bytes / (split_us * 1e-6) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(args.config, {}).get("bytes_per_launch")
+
+    result = {
+        "metric": "decode-attn achieved HBM GB/s (algorithmic bytes / time per call; µs/call alongside), "
+                  "Llama-3-8B shape b=32" if args.config == "llama3_8b_b32" else f"decode-attn achieved HBM GB/s, {args.config}",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "us_per_call": round(ms_per_step * 1e3, 2),
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if inp.cfg.kv_dtype == "bf16" else "fp8_e4m3 KV / bf16 q, fp32 softmax",
+        "data": "synthetic (seeded N(0,1) bf16 q/K/V generated on the CPU, resident in HBM before timing)",
+        "config": {
+            "workload": f"{args.config}: {inp.cfg.description}",
+            "algorithmic_bytes_per_call": alg_bytes,
+            "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
+            "kv_pools_rotated": len(pools),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": f"splitkv_{plan.algo}_kernel",
+            "achieved": round(split_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(split_gbps / HBM_PEAK_GBPS, 4),
+            "us_per_launch": round(split_us, 2),
+            "traffic": traffic,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(inp_cpu, args.cpu_seconds)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

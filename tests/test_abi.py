@@ -1,0 +1,203 @@
+"""C-ABI checks that need no GPU: the library loads, exports what include/fdk.h declares, the ctypes
+mirror has the C layout, and argument validation / planning work on fake pointers (dry run)."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fdk.h")
+
+from triton_distributed_amd import _lib  # noqa: E402
+from triton_distributed_amd._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkPlan  # noqa: E402
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fdk_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS), names
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.fdk_abi_version() == _lib.FDK_ABI_VERSION
+
+
+def test_ctypes_structs_match_the_c_layout(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "fdk.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
+         offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
+         offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes));
+  printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
+         offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
+  printf("%zu\n", sizeof(fdk_plan_t));
+  return 0;
+}''')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                   check=True)
+    lines = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
+    got = [int(x) for x in lines[0].split()]
+    want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
+                                       ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes")]
+    assert got == want
+    got = [int(x) for x in lines[1].split()]
+    want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
+                                             ("partial_lse", "kv_lens", "lse_stride_b_out")]
+    assert got == want
+    assert int(lines[2]) == C.sizeof(FdkPlan)
+
+
+def _args(**kw):
+    """A valid dry-run argument block on fake (never dereferenced) pointers: B32 32q/8kv P16 N4096."""
+    a = FdkDecodeArgs()
+    a.struct_size = C.sizeof(FdkDecodeArgs)
+    a.flags = _lib.FDK_FLAG_DRY_RUN
+    a.q, a.k_cache, a.v_cache = 0x10000, 0x20000, 0x30000
+    a.block_table, a.kv_lens, a.out, a.lse = 0x40000, 0x50000, 0x60000, 0x70000
+    a.q_dtype = a.kv_dtype = a.out_dtype = _lib.FDK_BF16
+    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim = 32, 32, 8, 128
+    a.page_size, a.max_pages = 16, 256
+    a.q_stride_b, a.q_stride_h = 32 * 128, 128
+    a.k_stride_page, a.k_stride_tok, a.k_stride_head = 16 * 8 * 128, 8 * 128, 128
+    a.v_stride_page, a.v_stride_tok, a.v_stride_head = 16 * 8 * 128, 8 * 128, 128
+    a.table_stride_b = 256
+    a.out_stride_b, a.out_stride_h = 32 * 128, 128
+    a.lse_stride_b = 32
+    a.sm_scale = 128 ** -0.5
+    a.workspace, a.workspace_bytes = 0x80000, 1 << 30
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+def _decode_rc(a):
+    return _lib.load().fdk_decode(C.byref(a), None)
+
+
+def test_valid_arguments_pass_dry_run():
+    assert _decode_rc(_args()) == 0
+    assert _lib.load().fdk_last_error() == b""
+
+
+@pytest.mark.parametrize("field,value,code", [
+    ("struct_size", 8, _lib.FDK_EABI),
+    ("q", None, _lib.FDK_ENULL),
+    ("kv_lens", None, _lib.FDK_ENULL),
+    ("out", None, _lib.FDK_ENULL),
+    ("q", 0x10008, _lib.FDK_EALIGN),
+    ("k_cache", 0x20004, _lib.FDK_EALIGN),
+    ("k_stride_tok", 8 * 128 + 4, _lib.FDK_EALIGN),
+    ("q_stride_h", 132, _lib.FDK_EALIGN),
+    ("num_kv_heads", 5, _lib.FDK_ESHAPE),
+    ("num_q_heads", 0, _lib.FDK_ESHAPE),
+    ("batch", -1, _lib.FDK_ESHAPE),
+    ("page_size", 0, _lib.FDK_ESHAPE),
+    ("max_pages", 0, _lib.FDK_ESHAPE),
+    ("table_stride_b", 255, _lib.FDK_ESHAPE),
+    ("out_stride_h", 127, _lib.FDK_ESHAPE),
+    ("num_splits", 5000, _lib.FDK_ESHAPE),
+    ("head_dim", 256, _lib.FDK_EUNSUPPORTED),
+    ("head_dim", 64, _lib.FDK_EUNSUPPORTED),
+    ("q_dtype", _lib.FDK_FP32, _lib.FDK_EUNSUPPORTED),
+    ("kv_dtype", _lib.FDK_FP16, _lib.FDK_EUNSUPPORTED),
+    ("out_dtype", _lib.FDK_FP8_E4M3, _lib.FDK_EUNSUPPORTED),
+    ("algo", 7, _lib.FDK_EUNSUPPORTED),
+    ("workspace", None, _lib.FDK_EWORKSPACE),
+    ("workspace_bytes", 1024, _lib.FDK_EWORKSPACE),
+    ("sm_scale", float("nan"), _lib.FDK_ESHAPE),
+])
+def test_bad_arguments_are_rejected_without_a_launch(field, value, code):
+    rc = _decode_rc(_args(**{field: value}))
+    assert rc == code, (_lib.load().fdk_last_error(), rc)
+    assert len(_lib.load().fdk_last_error()) > 0
+    with pytest.raises((ValueError, _lib.FdkError)):
+        _lib.check(rc)
+
+
+def test_packed_output_needs_a_wider_row():
+    a = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE)
+    assert _decode_rc(a) == _lib.FDK_ESHAPE
+    a = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE, out_stride_h=129, out_stride_b=32 * 129)
+    assert _decode_rc(a) == 0
+
+
+def test_null_args_and_empty_batch():
+    lib = _lib.load()
+    assert lib.fdk_decode(None, None) == _lib.FDK_ENULL
+    # an empty batch is a successful no-op even without the dry-run flag and with null tensors
+    a = _args(batch=0, flags=0, q=None, k_cache=None, out=None)
+    assert lib.fdk_decode(C.byref(a), None) == 0
+
+
+def _plan(a, cus=256):
+    p = FdkPlan()
+    rc = _lib.load().fdk_plan(C.byref(a), cus, C.byref(p))
+    assert rc == 0, _lib.load().fdk_last_error()
+    return p
+
+
+def test_plan_scales_splits_with_occupancy():
+    p = _plan(_args())                                    # 256 (b, kv head) units on 256 CUs
+    assert p.num_splits >= 2 and p.chunk_tokens % 64 == 0
+    assert p.num_splits * p.chunk_tokens >= 4096 > (p.num_splits - 1) * p.chunk_tokens
+    assert p.algo == _lib.FDK_ALGO_VALU                   # group 4: vector path
+    # few units, long context -> many splits; chunks never shorter than 256 tokens
+    p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
+                         q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
+    assert p_long.num_splits > p.num_splits and p_long.chunk_tokens >= 256
+    # huge batch -> no split at all
+    p_big = _plan(_args(batch=4096))
+    assert p_big.num_splits == 1
+    # short context is never split below the minimum chunk
+    p_short = _plan(_args(batch=1, max_pages=8, table_stride_b=8))
+    assert p_short.num_splits == 1 and p_short.chunk_tokens >= 128
+    # the host's bound on kv_len drives the split, not the table width
+    p_hint = _plan(_args(max_pages=2048, table_stride_b=2048, max_kv_len=4096))
+    assert (p_hint.num_splits, p_hint.chunk_tokens) == (p.num_splits, p.chunk_tokens)
+    # a forced split count is honoured and covers the whole range
+    p_forced = _plan(_args(num_splits=32))
+    assert p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
+    # fewer compute units -> fewer splits
+    assert _plan(_args(), cus=64).num_splits <= p.num_splits
+
+
+def test_workspace_bytes_formula():
+    lib = _lib.load()
+    assert lib.fdk_workspace_bytes(32, 32, 128, 4) >= 32 * 32 * 4 * 129 * 4
+    assert lib.fdk_workspace_bytes(32, 32, 128, 4) % 256 == 0
+    assert lib.fdk_workspace_bytes(0, 32, 128, 4) == 0
+    assert lib.fdk_workspace_bytes(32, 32, 128, 0) == 0
+
+
+def test_combine_ranks_validation():
+    lib = _lib.load()
+    a = FdkCombineRanksArgs()
+    a.struct_size = C.sizeof(FdkCombineRanksArgs)
+    a.flags = _lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE
+    a.partial, a.kv_lens, a.out = 0x1000, 0x2000, 0x3000
+    a.partial_dtype = a.out_dtype = _lib.FDK_BF16
+    a.num_ranks, a.batch, a.num_q_heads, a.head_dim = 8, 4, 32, 128
+    a.stride_r, a.stride_b, a.stride_h = 4 * 32 * 129, 32 * 129, 129
+    a.out_stride_b, a.out_stride_h = 32 * 128, 128
+    assert lib.fdk_combine_ranks(C.byref(a), None) == 0
+    a.stride_h = 128
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
+    a.stride_h = 129
+    a.flags = _lib.FDK_FLAG_DRY_RUN        # unpacked but no lse tensor
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ENULL
+    a.num_ranks = 0
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
+    assert lib.fdk_combine_ranks(None, None) == _lib.FDK_ENULL

@@ -1,0 +1,435 @@
+"""Parity of the HIP decode path with the oracle, on a real MI355X, through the C ABI.
+
+Tolerances (the bar this path is held to):
+  out  bf16/fp16: |out - ref| <= 2e-2 + 2e-2*|ref| against the torch restatement of the reference's
+       torch implementation, and a tighter 5e-3 + 1e-2*|x| against the exact float64 answer;
+  lse  fp32: |lse - lse64| <= 1e-3;
+  block_table indexing: bit-exact where the mathematics allows it (single-token sequences, page
+  permutations), no NaN/inf anywhere for kv_len >= 1."""
+import math
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
+
+import triton_distributed_amd as tda  # noqa: E402
+from triton_distributed_amd import workloads as wl  # noqa: E402
+from cases import EDGE_CASES, all_cases  # noqa: E402
+from oracle import closed_form as cf  # noqa: E402
+from oracle import fp8 as ofp8  # noqa: E402
+from oracle.paged_attn import ref_paged_attn  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+OUT_ATOL = OUT_RTOL = 2e-2
+LSE_ATOL = 1e-3
+GOLDEN = np.load(os.path.join(ROOT, "tests", "golden", "decode_golden.npz"))
+
+
+def _dev(c, device):
+    return {k: (v.to(device) if isinstance(v, torch.Tensor) else v) for k, v in c.items()}
+
+
+def _lens_t(lens, device):
+    return torch.as_tensor(list(lens), dtype=torch.int32, device=device)
+
+
+def _check(out, lse, q, k, v, table, lens, scale, soft_cap=0.0, k_scale=None, v_scale=None, ref_kv=None, tag=""):
+    """Compare one result with both oracles (run on the tensors' own device)."""
+    assert torch.isfinite(out.float()).all(), f"{tag}: non-finite out"
+    assert torch.isfinite(lse).all(), f"{tag}: non-finite lse"
+    rk, rv = ref_kv if ref_kv is not None else (k, v)
+    ref = ref_paged_attn(q, rk, rv, lens, table, scale, soft_cap)
+    torch.testing.assert_close(out.float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL, msg=lambda m: f"{tag} vs torch ref: {m}")
+    o64, l64 = cf.attn_fp64(q, rk, rv, table, lens, scale, soft_cap)
+    torch.testing.assert_close(out.double(), o64, atol=5e-3, rtol=1e-2, msg=lambda m: f"{tag} vs fp64: {m}")
+    torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0, msg=lambda m: f"{tag} lse: {m}")
+
+
+# ---- the reference's own test grid (test_decode_attn.py:123-162) ---------------------------------------------
+@pytest.mark.parametrize("kv_lens", [[1320, 18, 463], [1, 54, 293, 70]])
+@pytest.mark.parametrize("num_heads", [(16, 16), (32, 8), (64, 8), (6, 1)])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("soft_cap", [0, 30, 50])
+def test_reference_grid(cuda_device, kv_lens, num_heads, block_size, dtype, soft_cap):
+    print(f"case lens={kv_lens} heads={num_heads} P={block_size} {dtype} cap={soft_cap}", flush=True)
+    num_blocks = 1024
+    g = torch.Generator(device="cpu").manual_seed(hash((tuple(kv_lens), num_heads, block_size, soft_cap)) & 0xFFFF)
+    hq, hkv = num_heads
+    d = 128
+    scale = d ** -0.5
+    q = torch.randn(len(kv_lens), hq, d, generator=g).to(dtype).to(cuda_device)
+    kv = torch.randn(num_blocks + 1, 2, block_size, hkv, d, generator=g).to(dtype).to(cuda_device)
+    k, v = kv[:, 0], kv[:, 1]                       # strided views: page stride is twice the page extent
+    max_blocks = (max(kv_lens) + block_size - 1) // block_size
+    table = torch.randint(0, num_blocks, (len(kv_lens), max_blocks), generator=g, dtype=torch.int32).to(cuda_device)
+    lens_t = _lens_t(kv_lens, cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap))
+    torch.cuda.synchronize()
+    _check(out, lse, q, k, v, table, kv_lens, scale, float(soft_cap), tag="grid")
+    # the reference entry points: same numbers, reference layouts
+    o2 = tda.gqa_fwd_batch_decode(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale, float(soft_cap))
+    packed = tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale,
+                                                 float(soft_cap), kv_split=32)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, out)
+    assert packed.shape == (len(kv_lens), hq, d + 1) and packed.dtype == dtype
+    torch.testing.assert_close(packed[..., :d].float(), out.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(packed[..., d].float(), lse, atol=3e-2, rtol=1e-2)     # lse rounded to 16 bits
+
+
+def test_large_pool_index_arithmetic(cuda_device):
+    # NUM_BLOCKS = 32000 "large enough to test overflow in index calculation" (test_decode_attn.py:120):
+    # here the pool is made large enough that element offsets pass 2^31 and 2^32
+    hq, hkv, d, page = 32, 8, 128, 16
+    num_blocks = 140_000                       # 140000*16*8*128 = 2.29e9 elements (> 2^31), 4.6e9 bytes (> 2^32)
+    g = torch.Generator(device=cuda_device).manual_seed(5)
+    k = torch.randn(num_blocks, page, hkv, d, generator=g, device=cuda_device, dtype=torch.bfloat16)
+    v = torch.randn(num_blocks, page, hkv, d, generator=g, device=cuda_device, dtype=torch.bfloat16)
+    q = torch.randn(3, hq, d, generator=g, device=cuda_device, dtype=torch.bfloat16)
+    lens = [700, 16, 1]
+    table = torch.tensor([[num_blocks - 1 - 3 * i for i in range(44)],
+                          [num_blocks - 2] * 44, [70_000] * 44], dtype=torch.int32, device=cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5)
+    torch.cuda.synchronize()
+    _check(out, lse, q, k, v, table, lens, d ** -0.5, tag="bigpool")
+
+
+def test_head_dim_256_is_rejected(cuda_device):
+    q = torch.zeros(1, 8, 256, dtype=torch.float16, device=cuda_device)
+    k = torch.zeros(4, 16, 8, 256, dtype=torch.float16, device=cuda_device)
+    with pytest.raises(ValueError, match="head_dim"):
+        tda.flash_decode(q, k, k, torch.zeros(1, 1, dtype=torch.int32, device=cuda_device),
+                         _lens_t([1], cuda_device), 1.0)
+
+
+# ---- golden vectors and edge cases -----------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["tiny", *EDGE_CASES])
+@pytest.mark.parametrize("kv_split", [-1, 1, 3, 32])
+def test_golden_cases(cuda_device, name, kv_split):
+    print(f"case golden {name} kv_split={kv_split}", flush=True)
+    c = _dev(dict(all_cases())[name], cuda_device)
+    lens_t = _lens_t(c["kv_lens"], cuda_device)
+    out, lse = tda.flash_decode(c["q"], c["k_cache"], c["v_cache"], c["block_table"], lens_t, c["sm_scale"],
+                                soft_cap=c["soft_cap"], kv_split=kv_split)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    np.testing.assert_allclose(out.float().cpu().numpy(), GOLDEN[name + ".ref"], atol=OUT_ATOL, rtol=OUT_RTOL)
+    np.testing.assert_allclose(out.float().cpu().numpy(), GOLDEN[name + ".out64"], atol=5e-3, rtol=1e-2)
+    np.testing.assert_allclose(lse.cpu().numpy(), GOLDEN[name + ".lse64"], atol=LSE_ATOL, rtol=0)
+
+
+@pytest.mark.parametrize("page", [1, 16])
+def test_single_token_sequences_are_bit_exact_gathers(cuda_device, page):
+    g = torch.Generator().manual_seed(31)
+    b, hq, hkv, d, pool = 7, 8, 2, 128, 50
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.randint(0, pool, (b, 3), generator=g, dtype=torch.int32).to(cuda_device)
+    table[:, 1:] = 2**31 - 1                                       # never read
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t([1] * b, cuda_device), d ** -0.5)
+    torch.cuda.synchronize()
+    for i in range(b):
+        for h in range(hq):
+            assert torch.equal(out[i, h], v[table[i, 0].item(), 0, h // 4]), (i, h)   # softmax of one logit == 1
+            want = d ** -0.5 * float(torch.dot(q[i, h].double(), k[table[i, 0].item(), 0, h // 4].double()))
+            assert abs(float(lse[i, h]) - want) < 1e-4
+
+
+def test_zero_query_gives_mean_and_log_n(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["ragged_g8"], batch=9, kv_len_range=(1, 3000)), cuda_device,
+                         poison_tail=True)
+    q = torch.zeros_like(inp.q)
+    out, lse = tda.flash_decode(q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    torch.cuda.synchronize()
+    for b, n in enumerate(inp.kv_lens_host):
+        rows = cf.gather_kv(inp.v_cache, inp.block_table[b].cpu(), n).double()
+        torch.testing.assert_close(out[b].double(), rows[:, 0].mean(0).expand(8, -1), atol=2e-3, rtol=1e-2)
+        assert abs(float(lse[b, 0]) - math.log(n)) < 1e-4
+
+
+def test_rows_that_encode_their_slot_catch_a_wrong_gather(cuda_device):
+    # one sequence, V row r of the pool = r (spread over columns so that bf16 holds it exactly), K = 0:
+    # the output must be the exact mean of the slots named by block_table
+    page, hkv, d, pool = 16, 2, 128, 64
+    v = torch.zeros(pool, page, hkv, d)
+    idx = torch.arange(pool * page).view(pool, page)
+    v[:, :, 0, 0] = (idx % 256).float()
+    v[:, :, 0, 1] = (idx // 256).float()
+    v[:, :, 1, 2] = (idx % 256).float()
+    v[:, :, 1, 3] = (idx // 256).float()
+    v = v.to(torch.bfloat16).to(cuda_device)
+    k = torch.zeros_like(v)
+    q = torch.randn(1, 4, d).to(torch.bfloat16).to(cuda_device)
+    perm = torch.randperm(pool, generator=torch.Generator().manual_seed(1)).to(torch.int32)
+    n = 37 * page + 5
+    table = perm[None, :40].contiguous().to(cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t([n], cuda_device), 1.0, out=torch.empty(1, 4, d, device=cuda_device))
+    torch.cuda.synchronize()
+    slots = torch.cat([perm[i].item() * page + torch.arange(page) for i in range(38)])[:n].double()
+    lo, hi = (slots % 256).mean().item(), (slots // 256).float().mean().item()
+    got = out[0].double().cpu()
+    for h, (c0, c1) in enumerate([(0, 1), (0, 1), (2, 3), (2, 3)]):
+        assert abs(got[h, c0].item() - lo) < 0.5 and abs(got[h, c1].item() - hi) < 0.01, (h, got[h, :4], lo, hi)
+    assert abs(float(lse[0, 0]) - math.log(n)) < 1e-4
+
+
+def test_permuting_pool_pages_with_the_table_changes_nothing(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=1000), cuda_device)
+    out0, lse0 = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    pool = inp.k_cache.shape[0]
+    perm = torch.randperm(pool, generator=torch.Generator().manual_seed(9)).to(cuda_device)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(pool, device=cuda_device)
+    k2, v2 = inp.k_cache[perm], inp.v_cache[perm]                 # new page i holds old page perm[i]
+    table2 = inv[inp.block_table.long()].to(torch.int32)
+    out1, lse1 = tda.flash_decode(inp.q, k2, v2, table2, inp.kv_lens, inp.sm_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out0, out1) and torch.equal(lse0, lse1)
+
+
+def test_poisoned_table_tail_is_never_read(cuda_device):
+    cfg = wl.scaled_down(wl.CONFIGS["ragged_g8"], batch=12, kv_len_range=(1, 700))
+    a = wl.make_inputs(cfg, cuda_device, poison_tail=False)
+    b = wl.make_inputs(cfg, cuda_device, poison_tail=True)
+    assert not torch.equal(a.block_table, b.block_table)
+    oa, la = tda.flash_decode(a.q, a.k_cache, a.v_cache, a.block_table, a.kv_lens, a.sm_scale)
+    ob, lb = tda.flash_decode(b.q, b.k_cache, b.v_cache, b.block_table, b.kv_lens, b.sm_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(oa, ob) and torch.equal(la, lb)
+
+
+@pytest.mark.parametrize("kv_split", [32, 64])
+def test_short_sequences_and_empty_splits_stay_finite(cuda_device, kv_split):
+    lens = [1, 2, kv_split - 1, kv_split, kv_split + 1, 63, 64, 65, 255, 256, 257]
+    g = torch.Generator().manual_seed(77)
+    hq, hkv, d, page = 8, 2, 128, 16
+    pool = 200
+    q = torch.randn(len(lens), hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    # unused slots of live pages hold NaN: masked rows must not leak into the result
+    table = torch.randperm(pool, generator=g)[:len(lens) * 17].view(len(lens), 17).to(torch.int32).to(cuda_device)
+    for i, n in enumerate(lens):
+        last = table[i, (n - 1) // page].item()
+        if n % page:
+            k[last, n % page:] = float("nan")
+            v[last, n % page:] = float("nan")
+    # force real splitting of short sequences: pretend the host bound is the table width
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5, kv_split=kv_split)
+    torch.cuda.synchronize()
+    kc, vc = torch.nan_to_num(k), torch.nan_to_num(v)
+    _check(out, lse, q, kc, vc, table, lens, d ** -0.5, tag=f"short S={kv_split}")
+
+
+def test_split_invariance(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["ragged_g8"], batch=5, kv_len_range=(1, 9000)), cuda_device)
+    res = {}
+    for s in (1, 2, 3, 32, 64):
+        o = torch.empty(inp.q.shape, dtype=torch.float32, device=cuda_device)
+        res[s] = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                  kv_split=s, out=o)
+    torch.cuda.synchronize()
+    for s in (2, 3, 32, 64):
+        torch.testing.assert_close(res[s][0], res[1][0], atol=1e-3, rtol=5e-3)
+        torch.testing.assert_close(res[s][1], res[1][1], atol=2e-5, rtol=0)
+
+
+def test_zero_length_sequence_is_defined(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=300), cuda_device)
+    lens = _lens_t([300, 0, 17], cuda_device)
+    for s in (1, 4):
+        out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, lens, inp.sm_scale, kv_split=s)
+        torch.cuda.synchronize()
+        assert torch.all(out[1] == 0) and torch.all(torch.isneginf(lse[1]))
+        assert torch.isfinite(out[0].float()).all() and torch.isfinite(lse[[0, 2]]).all()
+
+
+def test_split_then_combine_entry_points_equal_the_fused_call(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=4, kv_len=2048), cuda_device)
+    for s in (1, 8):
+        ref_o, ref_l = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                        kv_split=s)
+        call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                  kv_split=s, always_workspace=True)
+        call.out.zero_()
+        call.run_splitkv()
+        torch.cuda.synchronize()
+        assert torch.all(call.out == 0)                     # the split entry point writes only the workspace
+        o, l = call.run_combine()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(o.float(), ref_o.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(l, ref_l, atol=1e-5, rtol=0)
+
+
+def test_runs_on_a_side_stream_and_is_repeatable(cuda_device):
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=4, kv_len=1500), cuda_device)
+    call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    o0, l0 = [t.clone() for t in call.run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            call.out.zero_()
+            o1, l1 = call.run()
+    side.synchronize()
+    assert torch.equal(o0, o1) and torch.equal(l0, l1)      # deterministic: no atomics, fixed merge order
+
+
+def test_inter_rank_combine_equals_one_shot(cuda_device):
+    # R ranks each hold a disjoint slice of every sequence (sequence parallel decode, one GPU stands in for all):
+    # local decode per rank -> packed [R,B,Hq,D+1] -> merge == decode over the whole sequence
+    r_, b, hq, hkv, d, page = 4, 3, 32, 8, 128, 16
+    g = torch.Generator().manual_seed(13)
+    shard_lens = torch.tensor([[512, 16, 0], [300, 0, 0], [0, 77, 0], [1, 1000, 5]], dtype=torch.int32)
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    pool = 80
+    ks = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
+    vs = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
+    tables = [torch.randperm(pool, generator=g)[:b * 21].view(b, 21).to(torch.int32).to(cuda_device) for _ in range(r_)]
+    packed = torch.full((r_, b, hq, d + 1), float("nan"), dtype=torch.float32, device=cuda_device)
+    outs = torch.empty(r_, b, hq, d, dtype=torch.bfloat16, device=cuda_device)
+    lses = torch.empty(r_, b, hq, dtype=torch.float32, device=cuda_device)
+    for r in range(r_):
+        lens_r = shard_lens[r].to(cuda_device)
+        o, l = tda.flash_decode(q, ks[r], vs[r], tables[r], lens_r, d ** -0.5, out=outs[r], lse=lses[r])
+        packed[r] = tda.pack_out_lse(o, l, torch.float32)
+        packed[r][(shard_lens[r] == 0).to(cuda_device)] = float("nan")   # what the reference leaves there
+    gl = shard_lens.to(cuda_device)
+    final = tda.inter_rank_combine(packed, gl)
+    final2 = tda.inter_rank_combine(outs, gl, all_ranks_lse=lses)
+    torch.cuda.synchronize()
+    # one-shot over the concatenation
+    for i in range(b):
+        kk = torch.cat([cf.gather_kv(ks[r], tables[r][i].cpu(), int(shard_lens[r, i])) for r in range(r_)])
+        vv = torch.cat([cf.gather_kv(vs[r], tables[r][i].cpu(), int(shard_lens[r, i])) for r in range(r_)])
+        n = kk.shape[0]
+        o64, _ = cf.attn_fp64(q[i:i + 1], kk[:, None].contiguous(), vv[:, None].contiguous(),
+                              torch.arange(n, dtype=torch.int32)[None], [n], d ** -0.5)
+        torch.testing.assert_close(final[i].double(), o64[0], atol=5e-3, rtol=1e-2)
+        torch.testing.assert_close(final2[i].double(), o64[0], atol=5e-3, rtol=1e-2)
+    # against the oracle's restatement of the reference merge
+    want = cf.combine_ranks(outs.cpu(), lses.cpu(), shard_lens)
+    torch.testing.assert_close(final2.double().cpu(), want, atol=4e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("page", [6, 24])
+def test_page_sizes_that_are_not_powers_of_two(cuda_device, page):
+    c = _dev(dict(all_cases())["odd_page6"], cuda_device) if page == 6 else None
+    if c is None:
+        g = torch.Generator().manual_seed(41)
+        lens = [500, 23, 24, 25]
+        pool = 60
+        c = dict(q=torch.randn(4, 8, 128, generator=g).to(torch.bfloat16).to(cuda_device),
+                 k_cache=torch.randn(pool, page, 2, 128, generator=g).to(torch.bfloat16).to(cuda_device),
+                 v_cache=torch.randn(pool, page, 2, 128, generator=g).to(torch.bfloat16).to(cuda_device),
+                 block_table=torch.randperm(pool, generator=g)[:4 * 21].view(4, 21).to(torch.int32).to(cuda_device),
+                 kv_lens=lens, sm_scale=128 ** -0.5, soft_cap=0.0)
+    out, lse = tda.flash_decode(c["q"], c["k_cache"], c["v_cache"], c["block_table"], _lens_t(c["kv_lens"], cuda_device),
+                                c["sm_scale"])
+    torch.cuda.synchronize()
+    _check(out, lse, c["q"], c["k_cache"], c["v_cache"], c["block_table"], c["kv_lens"], c["sm_scale"], tag=f"P={page}")
+
+
+# ---- fp8 KV cache ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("heads", [(32, 8), (64, 8), (8, 8)])
+def test_fp8_kv_cache_small(cuda_device, heads):
+    cfg = wl.DecodeConfig("fp8_small", 55, 5, heads[0], heads[1], 128, 16, kv_len_range=(1, 2000), kv_dtype="fp8_e4m3",
+                          spare_pages=4)
+    inp = wl.make_inputs(cfg, cuda_device, poison_tail=True)
+    out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                k_scale=inp.k_scale, v_scale=inp.v_scale)
+    torch.cuda.synchronize()
+    # the workload's definition: dequantise to bf16, then the same decode
+    kd = ofp8.dequant_per_head(inp.k_cache, inp.k_scale)
+    vd = ofp8.dequant_per_head(inp.v_cache, inp.v_scale)
+    _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
+           ref_kv=(kd, vd), tag="fp8")
+    # and, tighter, the exact dequantisation in float64 (no bf16 rounding of the scaled values)
+    o64, l64 = cf.attn_fp64(inp.q, inp.k_cache.float(), inp.v_cache.float(), inp.block_table, inp.kv_lens_host,
+                            inp.sm_scale, k_scale=inp.k_scale, v_scale=inp.v_scale)
+    torch.testing.assert_close(out.double(), o64, atol=5e-3, rtol=1e-2)
+    torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0)
+
+
+def test_fp8_every_byte_value_dequantises_exactly(cuda_device):
+    # 254 finite e4m3 codes as single-token V rows: out must equal table[code] * scale bit-exactly in fp32
+    table = torch.from_numpy(ofp8.e4m3fn_table())
+    codes = torch.tensor([c for c in range(256) if not math.isnan(table[c])], dtype=torch.uint8)
+    n = codes.numel()
+    v8 = codes.view(n, 1, 1, 1).expand(n, 1, 1, 128).contiguous().view(torch.float8_e4m3fn).to(cuda_device)
+    k8 = torch.zeros_like(v8)
+    q = torch.zeros(n, 1, 128, dtype=torch.bfloat16, device=cuda_device)
+    scale = torch.tensor([0.75], device=cuda_device)
+    bt = torch.arange(n, dtype=torch.int32, device=cuda_device)[:, None].contiguous()
+    out = torch.empty(n, 1, 128, dtype=torch.float32, device=cuda_device)
+    tda.flash_decode(q, k8, v8, bt, _lens_t([1] * n, cuda_device), 1.0, k_scale=scale, v_scale=scale, out=out)
+    torch.cuda.synchronize()
+    want = (table[codes.long()] * 0.75).to(cuda_device)
+    assert torch.equal(out[:, 0, 0], want) and torch.equal(out[:, 0, 127], want)
+
+
+# ---- the five benchmark configurations at full size ----------------------------------------------------------------
+def _full_config(name, cuda_device, lse_rows=None):
+    print(f"config {name}: generating", flush=True)
+    inp = wl.make_inputs(name, cuda_device)
+    print(f"config {name}: decode", flush=True)
+    out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                k_scale=inp.k_scale, v_scale=inp.v_scale)
+    torch.cuda.synchronize()
+    assert out.shape == inp.q.shape and out.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    return inp, out, lse
+
+
+def _check_rows(inp, out, lse, rows, tag):
+    """Oracle comparison on a subset of sequences (the oracle runs on the GPU tensors, one sequence at a time)."""
+    k, v = inp.k_cache, inp.v_cache
+    for b in rows:
+        sl = slice(b, b + 1)
+        lens = [inp.kv_lens_host[b]]
+        if inp.cfg.kv_dtype == "fp8_e4m3":
+            # dequantise only the pages this sequence uses
+            n_pg = (lens[0] + inp.cfg.page_size - 1) // inp.cfg.page_size
+            ids = inp.block_table[b, :n_pg].long()
+            kd = ofp8.dequant_per_head(k[ids], inp.k_scale)
+            vd = ofp8.dequant_per_head(v[ids], inp.v_scale)
+            tbl = torch.arange(n_pg, dtype=torch.int32, device=k.device)[None]
+            _check(out[sl], lse[sl], inp.q[sl], kd, vd, tbl, lens, inp.sm_scale, tag=f"{tag} b={b}")
+        else:
+            _check(out[sl], lse[sl], inp.q[sl], k, v, inp.block_table[sl], lens, inp.sm_scale, tag=f"{tag} b={b}")
+
+
+def test_config1_tiny(cuda_device):
+    inp, out, lse = _full_config("tiny", cuda_device)
+    assert out.shape == (2, 8, 128) and lse.shape == (2, 8)
+    _check_rows(inp, out, lse, range(2), "tiny")
+
+
+def test_config2_llama3_8b_b32(cuda_device):
+    inp, out, lse = _full_config("llama3_8b_b32", cuda_device)
+    _check_rows(inp, out, lse, range(32), "cfg2")
+
+
+def test_config3_ragged_g8(cuda_device):
+    inp, out, lse = _full_config("ragged_g8", cuda_device)
+    _check_rows(inp, out, lse, range(64), "cfg3")
+
+
+def test_config4_long_131k(cuda_device):
+    inp, out, lse = _full_config("long_131k", cuda_device)
+    _check_rows(inp, out, lse, range(4), "cfg4")
+
+
+def test_config5_fp8_70b_b128(cuda_device):
+    inp, out, lse = _full_config("fp8_70b_b128", cuda_device)
+    _check_rows(inp, out, lse, range(0, 128, 9), "cfg5")
+    # size-independent property at full size: the same sequence placed twice gives the same rows
+    assert torch.isfinite(out.float()).all()

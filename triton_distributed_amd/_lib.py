@@ -1,0 +1,121 @@
+"""ctypes binding of libfdk.so (declarations: include/fdk.h).
+
+The library is loaded from ``triton_distributed_amd/lib/libfdk.so``.  There is no fallback: if the file
+is missing or a symbol is absent, importing the decode entry points raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
+
+FDK_ABI_VERSION = 1
+
+# fdk_dtype
+FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
+# fdk_status
+FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK_EABI = 0, -1, -2, -3, -4, -5, -6
+# fdk_algo
+FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
+# flags
+FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN = 1, 2
+
+EXPORTS = (
+    "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
+    "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks",
+)
+
+
+class FdkPlan(C.Structure):
+    _fields_ = [("num_splits", C.c_int32), ("chunk_tokens", C.c_int32), ("algo", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
+class FdkDecodeArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("flags", C.c_uint32),
+        ("q", C.c_void_p), ("q_stride_b", C.c_int64), ("q_stride_h", C.c_int64), ("q_dtype", C.c_int32),
+        ("kv_dtype", C.c_int32), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("k_stride_page", C.c_int64), ("k_stride_tok", C.c_int64), ("k_stride_head", C.c_int64),
+        ("v_stride_page", C.c_int64), ("v_stride_tok", C.c_int64), ("v_stride_head", C.c_int64),
+        ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+        ("block_table", C.c_void_p), ("table_stride_b", C.c_int64), ("kv_lens", C.c_void_p),
+        ("batch", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("page_size", C.c_int32), ("max_pages", C.c_int32), ("max_kv_len", C.c_int32), ("num_splits", C.c_int32),
+        ("sm_scale", C.c_float), ("soft_cap", C.c_float),
+        ("out", C.c_void_p), ("out_stride_b", C.c_int64), ("out_stride_h", C.c_int64),
+        ("out_dtype", C.c_int32), ("algo", C.c_int32),
+        ("lse", C.c_void_p), ("lse_stride_b", C.c_int64),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class FdkCombineRanksArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("flags", C.c_uint32),
+        ("partial", C.c_void_p), ("stride_r", C.c_int64), ("stride_b", C.c_int64), ("stride_h", C.c_int64),
+        ("partial_dtype", C.c_int32), ("out_dtype", C.c_int32),
+        ("partial_lse", C.c_void_p), ("lse_stride_r", C.c_int64), ("lse_stride_b", C.c_int64),
+        ("kv_lens", C.c_void_p),
+        ("num_ranks", C.c_int32), ("batch", C.c_int32), ("num_q_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("out", C.c_void_p), ("out_stride_b", C.c_int64), ("out_stride_h", C.c_int64),
+        ("lse", C.c_void_p), ("lse_stride_b_out", C.c_int64),
+    ]
+
+
+class FdkError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"fdk error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load libfdk.so once and type its entry points.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = os.environ.get("FDK_LIBRARY", str(LIB_PATH))
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} not found: build it with `python -m triton_distributed_amd.build` (hipcc, gfx950). "
+            "There is no fallback implementation.")
+    lib = C.CDLL(path)
+    for name in EXPORTS:
+        if not hasattr(lib, name):
+            raise ImportError(f"{path} does not export {name}")
+    lib.fdk_abi_version.restype = C.c_int
+    lib.fdk_abi_version.argtypes = []
+    lib.fdk_last_error.restype = C.c_char_p
+    lib.fdk_last_error.argtypes = []
+    lib.fdk_device_cus.restype = C.c_int
+    lib.fdk_device_cus.argtypes = []
+    lib.fdk_plan.restype = C.c_int
+    lib.fdk_plan.argtypes = [C.POINTER(FdkDecodeArgs), C.c_int, C.POINTER(FdkPlan)]
+    lib.fdk_workspace_bytes.restype = C.c_size_t
+    lib.fdk_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
+    for name in ("fdk_decode", "fdk_decode_splitkv", "fdk_combine"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.POINTER(FdkDecodeArgs), C.c_void_p]
+    lib.fdk_combine_ranks.restype = C.c_int
+    lib.fdk_combine_ranks.argtypes = [C.POINTER(FdkCombineRanksArgs), C.c_void_p]
+    if lib.fdk_abi_version() != FDK_ABI_VERSION:
+        raise ImportError(f"{path}: ABI version {lib.fdk_abi_version()} != {FDK_ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    """Turn a non-zero return code into an exception carrying fdk_last_error()."""
+    if rc == 0:
+        return
+    msg = load().fdk_last_error().decode("utf-8", "replace")
+    if rc in (FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EABI):
+        raise ValueError(f"fdk: {msg} (code {rc})")
+    raise FdkError(rc, msg)

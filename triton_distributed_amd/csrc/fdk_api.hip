@@ -1,0 +1,352 @@
+// C ABI of the flash-decode kernels: argument validation, launch planning, dispatch.
+// Declarations and the reference interfaces they replace: include/fdk.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "fdk_device.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int elem_size(int dt) {
+    switch (dt) {
+        case FDK_BF16:
+        case FDK_FP16: return 2;
+        case FDK_FP8_E4M3: return 1;
+        case FDK_FP32: return 4;
+        default: return 0;
+    }
+}
+
+int ilog2_exact(int x) {
+    if (x <= 0 || (x & (x - 1)) != 0) return -1;
+    int s = 0;
+    while ((1 << s) < x) ++s;
+    return s;
+}
+
+int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Compute units of the current device; 256 (MI355X) when no device answers.
+int query_cus() {
+    static int cached[64] = {0};     // idempotent per-device cache; a race only repeats the query
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < 64) cached[dev] = n;
+    return n;
+}
+
+constexpr int kChunkAlign = 64;     // split boundaries fall on multiples of 64 tokens
+constexpr int kMinChunk = 256;      // never split finer than this
+constexpr int kMaxSplits = 1024;
+
+int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
+    if (!a) return fail(FDK_ENULL, "args is null");
+    if (a->struct_size != sizeof(fdk_decode_args))
+        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_decode_args));
+    if (a->batch < 0) return fail(FDK_ESHAPE, "batch %d < 0", a->batch);
+    if (a->num_q_heads <= 0 || a->num_kv_heads <= 0)
+        return fail(FDK_ESHAPE, "head counts must be positive (Hq=%d, Hkv=%d)", a->num_q_heads, a->num_kv_heads);
+    if (a->num_q_heads % a->num_kv_heads != 0)
+        return fail(FDK_ESHAPE, "Hq=%d not a multiple of Hkv=%d", a->num_q_heads, a->num_kv_heads);
+    if (a->head_dim != fdk::kHeadDim)
+        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (only %d)", a->head_dim, fdk::kHeadDim);
+    if (a->page_size <= 0) return fail(FDK_ESHAPE, "page_size %d <= 0", a->page_size);
+    if (a->max_pages <= 0) return fail(FDK_ESHAPE, "max_pages %d <= 0", a->max_pages);
+    if ((int64_t)a->max_pages * a->page_size > INT32_MAX)
+        return fail(FDK_ESHAPE, "max_pages*page_size overflows int32");
+    if (a->max_kv_len < 0) return fail(FDK_ESHAPE, "max_kv_len %d < 0", a->max_kv_len);
+    if (a->num_splits < 0 || a->num_splits > kMaxSplits)
+        return fail(FDK_ESHAPE, "num_splits %d outside [0, %d]", a->num_splits, kMaxSplits);
+    if (a->q_dtype != FDK_BF16 && a->q_dtype != FDK_FP16)
+        return fail(FDK_EUNSUPPORTED, "q_dtype %d (bf16 or fp16 only)", a->q_dtype);
+    if (a->kv_dtype != a->q_dtype && a->kv_dtype != FDK_FP8_E4M3)
+        return fail(FDK_EUNSUPPORTED, "kv_dtype %d must equal q_dtype or be fp8_e4m3", a->kv_dtype);
+    if (a->algo < FDK_ALGO_AUTO || a->algo > FDK_ALGO_MFMA) return fail(FDK_EUNSUPPORTED, "algo %d", a->algo);
+    if (!(a->sm_scale == a->sm_scale)) return fail(FDK_ESHAPE, "sm_scale is NaN");
+    if (a->batch == 0) return FDK_OK;
+
+    if (!a->q || !a->k_cache || !a->v_cache || !a->block_table || !a->kv_lens)
+        return fail(FDK_ENULL, "q / k_cache / v_cache / block_table / kv_lens must be non-null");
+    if (!aligned16(a->q) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+        return fail(FDK_EALIGN, "q, k_cache and v_cache must be 16-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(a->block_table) & 3u) || (reinterpret_cast<uintptr_t>(a->kv_lens) & 3u))
+        return fail(FDK_EALIGN, "block_table / kv_lens must be 4-byte aligned");
+    const int kes = elem_size(a->kv_dtype);
+    if ((a->q_stride_b * 2) % 16 || (a->q_stride_h * 2) % 16)
+        return fail(FDK_EALIGN, "q strides must be multiples of 16 bytes");
+    const int64_t ks[6] = {a->k_stride_page, a->k_stride_tok, a->k_stride_head,
+                           a->v_stride_page, a->v_stride_tok, a->v_stride_head};
+    for (int i = 0; i < 6; ++i) {
+        if (ks[i] < 0) return fail(FDK_ESHAPE, "negative cache stride");
+        if ((ks[i] * kes) % 16) return fail(FDK_EALIGN, "cache strides must be multiples of 16 bytes");
+    }
+    if (a->k_stride_head < fdk::kHeadDim && a->num_kv_heads > 1)
+        return fail(FDK_ESHAPE, "k head stride %lld < head_dim", (long long)a->k_stride_head);
+    if (a->table_stride_b < a->max_pages)
+        return fail(FDK_ESHAPE, "table_stride_b %lld < max_pages %d", (long long)a->table_stride_b, a->max_pages);
+
+    if (need_out) {
+        if (!a->out) return fail(FDK_ENULL, "out is null");
+        const int oes = elem_size(a->out_dtype);
+        if (a->out_dtype != FDK_BF16 && a->out_dtype != FDK_FP16 && a->out_dtype != FDK_FP32)
+            return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);
+        if (reinterpret_cast<uintptr_t>(a->out) % oes) return fail(FDK_EALIGN, "out not element aligned");
+        const int row = fdk::kHeadDim + ((a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0);
+        if (a->out_stride_h < row) return fail(FDK_ESHAPE, "out_stride_h %lld < %d", (long long)a->out_stride_h, row);
+        if (a->lse && (reinterpret_cast<uintptr_t>(a->lse) & 3u)) return fail(FDK_EALIGN, "lse not 4-byte aligned");
+        if (a->lse && a->lse_stride_b < a->num_q_heads)
+            return fail(FDK_ESHAPE, "lse_stride_b %lld < Hq", (long long)a->lse_stride_b);
+    }
+    (void)need_workspace_only;
+    return FDK_OK;
+}
+
+int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
+    const int group = a->num_q_heads / a->num_kv_heads;
+    int algo = a->algo;
+    if (algo == FDK_ALGO_AUTO) {
+        // Matrix cores only where the q-head group makes a real tile (>= 8 heads per kv head).
+        algo = (group >= 8 && fdk::mfma_supported(a->q_dtype, a->kv_dtype, group)) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
+    }
+    if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group))
+        return fail(FDK_EUNSUPPORTED, "MFMA path not built for q_dtype=%d kv_dtype=%d group=%d", a->q_dtype,
+                    a->kv_dtype, group);
+    if (algo == FDK_ALGO_VALU && !fdk::valu_supported(a->q_dtype, a->kv_dtype, group))
+        return fail(FDK_EUNSUPPORTED, "VALU path not built for q_dtype=%d kv_dtype=%d", a->q_dtype, a->kv_dtype);
+
+    int64_t max_len = a->max_kv_len > 0 ? a->max_kv_len : (int64_t)a->max_pages * a->page_size;
+    const int64_t table_cap = (int64_t)a->max_pages * a->page_size;
+    if (max_len > table_cap) max_len = table_cap;
+    if (max_len < 1) max_len = 1;
+
+    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group) : fdk::valu_heads_per_wg(group);
+    const int head_tiles = (group + hpw - 1) / hpw;
+    const int64_t units = (int64_t)(a->batch > 0 ? a->batch : 1) * a->num_kv_heads * head_tiles;
+
+    int64_t splits;
+    if (a->num_splits > 0) {
+        splits = a->num_splits;
+    } else {
+        if (num_cus <= 0) num_cus = query_cus();
+        // Aim at ~8 workgroups (32 wavefronts) per compute unit, but keep chunks >= kMinChunk tokens.
+        const int64_t target = (int64_t)num_cus * 8;
+        splits = cdiv64(target, units);
+        const int64_t cap = cdiv64(max_len, kMinChunk);
+        if (splits > cap) splits = cap;
+        if (splits < 1) splits = 1;
+    }
+    int64_t chunk = cdiv64(cdiv64(max_len, splits), kChunkAlign) * kChunkAlign;
+    if (a->num_splits <= 0) splits = cdiv64(max_len, chunk);   // drop splits that would always be empty
+    if (splits > kMaxSplits) {
+        splits = kMaxSplits;
+        chunk = cdiv64(cdiv64(max_len, splits), kChunkAlign) * kChunkAlign;
+    }
+    plan->num_splits = (int32_t)splits;
+    plan->chunk_tokens = (int32_t)chunk;
+    plan->algo = algo;
+    plan->reserved = head_tiles;
+    return FDK_OK;
+}
+
+struct Resolved {
+    fdk_plan_t plan;
+    fdk::SplitParams sp;
+    fdk::CombineParams cp;
+};
+
+int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
+    int rc = make_plan(a, 0, &r->plan);
+    if (rc) return rc;
+    const int S = r->plan.num_splits;
+    const bool direct = direct_ok && S == 1;
+    const int64_t rows = (int64_t)a->batch * a->num_q_heads;
+    if ((int64_t)a->batch * S * a->num_kv_heads * r->plan.reserved > INT32_MAX)
+        return fail(FDK_ESHAPE, "grid too large");
+    float* part_o = nullptr;
+    float* part_lse = nullptr;
+    if (!direct && a->batch > 0) {
+        const size_t need = fdk_workspace_bytes(a->batch, a->num_q_heads, a->head_dim, S);
+        if (!a->workspace) return fail(FDK_EWORKSPACE, "workspace is null; %zu bytes needed", need);
+        if (!aligned16(a->workspace)) return fail(FDK_EALIGN, "workspace must be 16-byte aligned");
+        if (a->workspace_bytes < need)
+            return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed for %d splits", a->workspace_bytes, need, S);
+        part_o = reinterpret_cast<float*>(a->workspace);
+        part_lse = part_o + rows * S * fdk::kHeadDim;
+    }
+    fdk::SplitParams& sp = r->sp;
+    memset(&sp, 0, sizeof(sp));
+    sp.q = a->q; sp.k = a->k_cache; sp.v = a->v_cache;
+    sp.block_table = a->block_table; sp.kv_lens = a->kv_lens;
+    sp.k_scale = a->kv_dtype == FDK_FP8_E4M3 ? a->k_scale : nullptr;
+    sp.v_scale = a->kv_dtype == FDK_FP8_E4M3 ? a->v_scale : nullptr;
+    sp.part_o = part_o; sp.part_lse = part_lse;
+    sp.out = a->out; sp.lse = a->lse;
+    sp.q_sb = a->q_stride_b; sp.q_sh = a->q_stride_h;
+    sp.k_sp = a->k_stride_page; sp.k_st = a->k_stride_tok; sp.k_sh = a->k_stride_head;
+    sp.v_sp = a->v_stride_page; sp.v_st = a->v_stride_tok; sp.v_sh = a->v_stride_head;
+    sp.tbl_sb = a->table_stride_b;
+    sp.out_sb = a->out_stride_b; sp.out_sh = a->out_stride_h; sp.lse_sb = a->lse_stride_b;
+    sp.batch = a->batch; sp.hq = a->num_q_heads; sp.hkv = a->num_kv_heads;
+    sp.group = a->num_q_heads / a->num_kv_heads;
+    sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
+    sp.num_splits = S; sp.chunk = r->plan.chunk_tokens;
+    sp.head_tiles = r->plan.reserved;
+    sp.out_dtype = a->out_dtype;
+    sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
+    sp.direct = direct ? 1 : 0;
+    sp.scale_log2 = a->sm_scale * fdk::kLog2e;
+    sp.soft_cap = a->soft_cap > 0.f ? a->soft_cap : 0.f;
+    sp.sm_scale = a->sm_scale;
+
+    fdk::CombineParams& cp = r->cp;
+    memset(&cp, 0, sizeof(cp));
+    cp.part_o = part_o; cp.part_lse = part_lse; cp.kv_lens = a->kv_lens;
+    cp.out = a->out; cp.lse = a->lse;
+    cp.out_sb = a->out_stride_b; cp.out_sh = a->out_stride_h; cp.lse_sb = a->lse_stride_b;
+    cp.batch = a->batch; cp.hq = a->num_q_heads;
+    cp.num_splits = S; cp.chunk = r->plan.chunk_tokens;
+    cp.out_dtype = a->out_dtype; cp.pack_lse = sp.pack_lse;
+    return FDK_OK;
+}
+
+int launch_split(const fdk_decode_args* a, const Resolved& r, hipStream_t stream) {
+    int rc = r.plan.algo == FDK_ALGO_MFMA ? fdk::launch_splitkv_mfma(r.sp, a->q_dtype, a->kv_dtype, stream)
+                                          : fdk::launch_splitkv_valu(r.sp, a->q_dtype, a->kv_dtype, stream);
+    if (rc) return fail(rc, "split kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fdk_abi_version(void) { return FDK_ABI_VERSION; }
+
+const char* fdk_last_error(void) { return g_err; }
+
+int fdk_device_cus(void) { return query_cus(); }
+
+size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim, int32_t num_splits) {
+    if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 0) return 0;
+    const size_t rows = (size_t)batch * (size_t)num_q_heads * (size_t)num_splits;
+    size_t bytes = rows * ((size_t)head_dim + 1) * sizeof(float);
+    return (bytes + 255) & ~(size_t)255;
+}
+
+int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
+    g_err[0] = 0;
+    if (!plan) return fail(FDK_ENULL, "plan is null");
+    int rc = validate(args, false, false);
+    if (rc) return rc;
+    if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = 256;
+    return make_plan(args, num_cus, plan);
+}
+
+int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = validate(args, true, false);
+    if (rc) return rc;
+    if (args->flags & FDK_FLAG_DRY_RUN) {
+        fdk_plan_t plan;
+        rc = make_plan(args, 256, &plan);
+        if (rc) return rc;
+        if (plan.num_splits > 1 && args->batch > 0) {
+            const size_t need = fdk_workspace_bytes(args->batch, args->num_q_heads, args->head_dim, plan.num_splits);
+            if (!args->workspace) return fail(FDK_EWORKSPACE, "workspace is null; %zu bytes needed", need);
+            if (args->workspace_bytes < need)
+                return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed", args->workspace_bytes, need);
+        }
+        return FDK_OK;
+    }
+    if (args->batch == 0) return FDK_OK;
+    Resolved r;
+    rc = resolve(args, true, &r);
+    if (rc) return rc;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    rc = launch_split(args, r, stream);
+    if (rc) return rc;
+    if (!r.sp.direct) {
+        rc = fdk::launch_combine(r.cp, stream);
+        if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    }
+    return FDK_OK;
+}
+
+int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = validate(args, false, true);
+    if (rc) return rc;
+    if (args->batch == 0 || (args->flags & FDK_FLAG_DRY_RUN)) return FDK_OK;
+    Resolved r;
+    rc = resolve(args, false, &r);
+    if (rc) return rc;
+    return launch_split(args, r, reinterpret_cast<hipStream_t>(hip_stream));
+}
+
+int fdk_combine(const fdk_decode_args* args, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = validate(args, true, true);
+    if (rc) return rc;
+    if (args->batch == 0 || (args->flags & FDK_FLAG_DRY_RUN)) return FDK_OK;
+    Resolved r;
+    rc = resolve(args, false, &r);
+    if (rc) return rc;
+    rc = fdk::launch_combine(r.cp, reinterpret_cast<hipStream_t>(hip_stream));
+    if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
+int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
+    g_err[0] = 0;
+    if (!a) return fail(FDK_ENULL, "args is null");
+    if (a->struct_size != sizeof(fdk_combine_ranks_args))
+        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_combine_ranks_args));
+    if (a->num_ranks <= 0 || a->batch < 0 || a->num_q_heads <= 0)
+        return fail(FDK_ESHAPE, "bad dims R=%d B=%d Hq=%d", a->num_ranks, a->batch, a->num_q_heads);
+    if (a->head_dim != fdk::kHeadDim) return fail(FDK_EUNSUPPORTED, "head_dim %d not built", a->head_dim);
+    const bool packed = (a->flags & FDK_FLAG_PACK_LSE) != 0;
+    if (elem_size(a->partial_dtype) < 2) return fail(FDK_EUNSUPPORTED, "partial_dtype %d", a->partial_dtype);
+    if (elem_size(a->out_dtype) < 2) return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);
+    if (a->batch == 0) return FDK_OK;
+    if (!a->partial || !a->kv_lens || !a->out) return fail(FDK_ENULL, "partial / kv_lens / out must be non-null");
+    if (!packed && !a->partial_lse) return fail(FDK_ENULL, "partial_lse is null and FDK_FLAG_PACK_LSE is not set");
+    if (a->stride_h < fdk::kHeadDim + (packed ? 1 : 0)) return fail(FDK_ESHAPE, "stride_h too small");
+    if (a->out_stride_h < fdk::kHeadDim) return fail(FDK_ESHAPE, "out_stride_h too small");
+    if (a->flags & FDK_FLAG_DRY_RUN) return FDK_OK;
+    fdk::CombineRanksParams p;
+    memset(&p, 0, sizeof(p));
+    p.partial = a->partial; p.partial_lse = a->partial_lse; p.kv_lens = a->kv_lens;
+    p.out = a->out; p.lse = a->lse;
+    p.stride_r = a->stride_r; p.stride_b = a->stride_b; p.stride_h = a->stride_h;
+    p.lse_stride_r = a->lse_stride_r; p.lse_stride_b = a->lse_stride_b;
+    p.out_sb = a->out_stride_b; p.out_sh = a->out_stride_h; p.lse_sb_out = a->lse_stride_b_out;
+    p.num_ranks = a->num_ranks; p.batch = a->batch; p.hq = a->num_q_heads;
+    p.partial_dtype = a->partial_dtype; p.out_dtype = a->out_dtype; p.packed = packed ? 1 : 0;
+    int rc = fdk::launch_combine_ranks(p, reinterpret_cast<hipStream_t>(hip_stream));
+    if (rc) return fail(rc, "rank combine launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
+}  // extern "C"

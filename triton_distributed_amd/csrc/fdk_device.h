@@ -1,0 +1,179 @@
+// Shared device-side definitions for the flash-decode kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fdk.h"
+
+namespace fdk {
+
+constexpr int kHeadDim = 128;       // the only head dimension built
+constexpr int kWaveSize = 64;
+constexpr int kWavesPerWg = 4;      // split kernels run 256-thread workgroups
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Kernel arguments of the split kernels (passed by value).
+struct SplitParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const int32_t* block_table;
+    const int32_t* kv_lens;
+    const float* k_scale;
+    const float* v_scale;
+    float* part_o;    // [B, Hq, S, D] fp32 (S > 1)
+    float* part_lse;  // [B, Hq, S]    fp32 (S > 1)
+    void* out;        // final output, written directly when S == 1
+    float* lse;       // may be null
+    int64_t q_sb, q_sh;
+    int64_t k_sp, k_st, k_sh;  // page / token / head strides, elements
+    int64_t v_sp, v_st, v_sh;
+    int64_t tbl_sb;
+    int64_t out_sb, out_sh, lse_sb;
+    int32_t batch, hq, hkv, group;
+    int32_t page_size, page_shift;  // page_shift = log2(page_size) or -1
+    int32_t num_splits, chunk;
+    int32_t head_tiles;             // ceil(group / heads-per-workgroup)
+    int32_t out_dtype;              // fdk_dtype
+    int32_t pack_lse;
+    int32_t direct;                 // 1: single split, write the final (out, lse) instead of partials
+    float scale_log2;               // sm_scale * log2(e)
+    float soft_cap;                 // > 0: on (applied to natural-unit logits)
+    float sm_scale;
+};
+
+struct CombineParams {
+    const float* part_o;
+    const float* part_lse;
+    const int32_t* kv_lens;
+    void* out;
+    float* lse;
+    int64_t out_sb, out_sh, lse_sb;
+    int32_t batch, hq;
+    int32_t num_splits, chunk;
+    int32_t out_dtype;
+    int32_t pack_lse;
+};
+
+struct CombineRanksParams {
+    const void* partial;
+    const float* partial_lse;
+    const int32_t* kv_lens;
+    void* out;
+    float* lse;
+    int64_t stride_r, stride_b, stride_h;
+    int64_t lse_stride_r, lse_stride_b;
+    int64_t out_sb, out_sh, lse_sb_out;
+    int32_t num_ranks, batch, hq;
+    int32_t partial_dtype, out_dtype, packed;
+};
+
+// Launchers implemented in the .hip files; return hipError_t as int.
+int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
+int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
+int launch_combine(const CombineParams& p, hipStream_t stream);
+int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
+bool valu_supported(int q_dtype, int kv_dtype, int group);
+bool mfma_supported(int q_dtype, int kv_dtype, int group);
+int valu_heads_per_wg(int group);
+int mfma_heads_per_wg(int group);
+
+#if defined(__HIPCC__)
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over aligned groups of LANES lanes (LANES in {4, 8, 16}); every lane of the group gets the total.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float x) {
+    x += dpp_mov<0xB1>(x);                 // quad_perm [1,0,3,2]
+    x += dpp_mov<0x4E>(x);                 // quad_perm [2,3,0,1]
+    if (LANES >= 8) x += dpp_mov<0x141>(x);   // row_half_mirror
+    if (LANES >= 16) x += dpp_mov<0x140>(x);  // row_mirror
+    return x;
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+    return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// soft cap: cap * tanh(x / cap), tanh(y) = 1 - 2 / (exp(2y) + 1)
+__device__ __forceinline__ float soft_cap_fn(float x, float cap, float inv_cap) {
+    float e = fast_exp2(2.0f * kLog2e * x * inv_cap);
+    return cap * (1.0f - 2.0f * fast_rcp(e + 1.0f));
+}
+
+// dtype helpers -----------------------------------------------------------------------------------
+template <int DT> struct Pack2;  // two 16-bit floats in a dword
+template <> struct Pack2<FDK_BF16> {
+    using vec = bf16x2_t;
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(vec, a), __builtin_bit_cast(vec, b), c, false);
+    }
+    static __device__ __forceinline__ float lo(uint32_t a) { return __builtin_bit_cast(float, a << 16); }
+    static __device__ __forceinline__ float hi(uint32_t a) { return __builtin_bit_cast(float, a & 0xffff0000u); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        vec r = {(__bf16)a, (__bf16)b};
+        return __builtin_bit_cast(uint32_t, r);
+    }
+    static __device__ __forceinline__ uint32_t from_fp8_lo(uint32_t w) {  // bytes 0,1 -> two bf16
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+    }
+    static __device__ __forceinline__ uint32_t from_fp8_hi(uint32_t w) {  // bytes 2,3
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+    }
+};
+template <> struct Pack2<FDK_FP16> {
+    using vec = f16x2_t;
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(vec, a), __builtin_bit_cast(vec, b), c, false);
+    }
+    static __device__ __forceinline__ float lo(uint32_t a) { return (float)__builtin_bit_cast(vec, a).x; }
+    static __device__ __forceinline__ float hi(uint32_t a) { return (float)__builtin_bit_cast(vec, a).y; }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        vec r = {(_Float16)a, (_Float16)b};
+        return __builtin_bit_cast(uint32_t, r);
+    }
+    static __device__ __forceinline__ uint32_t from_fp8_lo(uint32_t w) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+    }
+    static __device__ __forceinline__ uint32_t from_fp8_hi(uint32_t w) {
+        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+    }
+};
+
+// Store one output element in the requested dtype.
+__device__ __forceinline__ void store_out(void* base, int64_t idx, float x, int dtype) {
+    if (dtype == FDK_BF16) {
+        reinterpret_cast<__bf16*>(base)[idx] = (__bf16)x;
+    } else if (dtype == FDK_FP16) {
+        reinterpret_cast<_Float16*>(base)[idx] = (_Float16)x;
+    } else {
+        reinterpret_cast<float*>(base)[idx] = x;
+    }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace fdk

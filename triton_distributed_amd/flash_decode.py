@@ -1,0 +1,369 @@
+"""Host side of the MI355X flash-decode path: split-KV paged GQA decode + LSE combine.
+
+Mirrors the operator interface of the reference's
+``python/triton_dist/kernels/nvidia/flash_decode.py`` for this one path:
+
+=====================================  =========================================================
+here                                   reference
+=====================================  =========================================================
+``flash_decode``                       the local step of ``SpGQAFlashDecodeAttention.forward``
+                                       (layers/nvidia/sp_flash_decode_layer.py:100-110), returned
+                                       as ``(out, lse)`` instead of the packed buffer
+``gqa_fwd_batch_decode_intra_rank``    flash_decode.py:847-928  (packed ``[B, Hq, D+1]``)
+``gqa_fwd_batch_decode``               flash_decode.py:763-844  (``[B, Hq, D]``)
+``*_aot`` variants                     flash_decode.py:979-1092 (explicit stream first)
+``inter_rank_combine``                 the final combine of sp_flash_decode_layer.py:143-183 with
+                                       kernel flash_decode.py:481-532
+``get_split_kv_plan``                  ``get_triton_split_kv_algo_info``, flash_decode.py:103-109
+``pack_out_lse`` / ``unpack_out_lse``  the ``[..., :D]`` / ``[..., D]`` layout of :235-239, :441-449
+=====================================  =========================================================
+
+Same names, argument order and meaning; the kernels behind them are hand-written gfx950 HIP kernels in
+``libfdk.so`` reached through its C ABI (include/fdk.h).  torch only supplies device memory and the
+current stream.  There is no fallback path: a missing library raises at import of this module.
+
+Differences that a caller can observe
+  * the split count defaults to a value chosen from the shape and the device's compute units
+    (reference: fixed 32, :863); ``kv_split`` still forces a count;
+  * the per-split scratch is fp32 and private to the library: a caller-provided ``output_split`` is used
+    as scratch only if it is large enough, its contents afterwards are unspecified;
+  * ``workspace`` and ``q_lens`` are accepted and ignored, exactly as in the reference (:847, never read);
+  * kv_len == 0 gives out = 0, lse = -inf instead of NaN.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Sequence, Tuple, Union
+
+import torch
+
+from . import _lib
+from ._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkPlan
+
+_LIB = _lib.load()          # raises ImportError when libfdk.so is not built - by design
+
+_TORCH_TO_FDK = {torch.bfloat16: _lib.FDK_BF16, torch.float16: _lib.FDK_FP16, torch.float32: _lib.FDK_FP32}
+if hasattr(torch, "float8_e4m3fn"):
+    _TORCH_TO_FDK[torch.float8_e4m3fn] = _lib.FDK_FP8_E4M3
+_ALGOS = {"auto": _lib.FDK_ALGO_AUTO, "valu": _lib.FDK_ALGO_VALU, "mfma": _lib.FDK_ALGO_MFMA}
+_ALGO_NAMES = {v: k for k, v in _ALGOS.items()}
+
+
+def _fdk_dtype(t: torch.dtype, what: str) -> int:
+    try:
+        return _TORCH_TO_FDK[t]
+    except KeyError:
+        raise ValueError(f"{what}: unsupported dtype {t}") from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream_handle(stream) -> int:
+    if stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if isinstance(stream, int):
+        return stream
+    return stream.cuda_stream
+
+
+@dataclass
+class SplitKvPlan:
+    """Shape-dependent launch constants (the role of the reference's ``algo_info`` dict)."""
+    num_splits: int
+    chunk_tokens: int
+    algo: str
+    workspace_bytes: int
+
+
+def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
+               k_scale, v_scale, algo, check_device=True) -> FdkDecodeArgs:
+    if q.dim() != 3:
+        raise ValueError(f"q must be [batch, q_heads, head_dim], got {tuple(q.shape)}")
+    if k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise ValueError("k_cache / v_cache must be [num_pages, page_size, kv_heads, head_dim]")
+    batch, q_heads, q_head_dim = q.shape
+    _, page_size, kv_heads, k_head_dim = k_cache.shape
+    # the reference's shape asserts, flash_decode.py:851,860
+    assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
+    assert q_heads % kv_heads == 0
+    if v_cache.shape[-1] != q_head_dim:
+        raise ValueError(f"v head_dim {v_cache.shape[-1]} != q head_dim {q_head_dim} is not built")
+    if k_cache.dtype != v_cache.dtype:
+        raise ValueError("k_cache and v_cache must share a dtype")
+    if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:
+        raise ValueError("the head dimension of q, k_cache and v_cache must be contiguous")
+    if block_table.dim() != 2 or block_table.shape[0] != batch:
+        raise ValueError(f"block_table must be [batch, max_pages], got {tuple(block_table.shape)}")
+    if block_table.dtype != torch.int32 or kv_lens.dtype != torch.int32:
+        raise ValueError("block_table and kv_lens must be int32")
+    if block_table.stride(-1) != 1 or (kv_lens.dim() != 1 or kv_lens.shape[0] != batch or
+                                       (batch > 1 and kv_lens.stride(0) != 1)):
+        raise ValueError("block_table rows and kv_lens [batch] must be contiguous")
+    if check_device:
+        for name, t in (("q", q), ("k_cache", k_cache), ("v_cache", v_cache), ("block_table", block_table),
+                        ("kv_lens", kv_lens)):
+            if not t.is_cuda:
+                raise ValueError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+            if t.device != q.device:
+                raise ValueError(f"{name} is on {t.device}, q on {q.device}")
+    a = FdkDecodeArgs()
+    a.struct_size = C.sizeof(FdkDecodeArgs)
+    a.flags = 0
+    a.q = q.data_ptr()
+    a.q_stride_b, a.q_stride_h = q.stride(0), q.stride(1)
+    a.q_dtype = _fdk_dtype(q.dtype, "q")
+    a.kv_dtype = _fdk_dtype(k_cache.dtype, "k_cache")
+    a.k_cache, a.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+    a.k_stride_page, a.k_stride_tok, a.k_stride_head = k_cache.stride(0), k_cache.stride(1), k_cache.stride(2)
+    a.v_stride_page, a.v_stride_tok, a.v_stride_head = v_cache.stride(0), v_cache.stride(1), v_cache.stride(2)
+    if a.kv_dtype == _lib.FDK_FP8_E4M3:
+        for name, s in (("k_scale", k_scale), ("v_scale", v_scale)):
+            if s is not None and (s.dtype != torch.float32 or s.numel() != kv_heads or not s.is_contiguous()):
+                raise ValueError(f"{name} must be a contiguous fp32 tensor of {kv_heads} per-kv-head scales")
+        a.k_scale, a.v_scale = _ptr(k_scale), _ptr(v_scale)
+    elif k_scale is not None or v_scale is not None:
+        raise ValueError("k_scale / v_scale are only meaningful for an fp8 KV cache")
+    a.block_table = block_table.data_ptr()
+    a.table_stride_b = block_table.stride(0) if batch > 1 else max(block_table.stride(0), block_table.shape[1])
+    a.kv_lens = kv_lens.data_ptr()
+    a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim = batch, q_heads, kv_heads, q_head_dim
+    a.page_size = page_size
+    a.max_pages = block_table.shape[1]
+    a.max_kv_len = int(max_kv_len) if max_kv_len else 0
+    a.num_splits = int(kv_split) if kv_split and kv_split > 0 else 0
+    a.sm_scale = float(sm_scale)
+    a.soft_cap = float(soft_cap) if soft_cap else 0.0
+    a.algo = _ALGOS[algo] if isinstance(algo, str) else int(algo)
+    return a
+
+
+def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
+    plan = FdkPlan()
+    _lib.check(_LIB.fdk_plan(C.byref(a), num_cus, C.byref(plan)))
+    ws = _LIB.fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits)
+    return SplitKvPlan(plan.num_splits, plan.chunk_tokens, _ALGO_NAMES[plan.algo], int(ws))
+
+
+def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, soft_cap=0.0, kv_split=-1,
+                      max_kv_len=None, algo="auto", num_cus: int = 0) -> SplitKvPlan:
+    """The split count / chunk length / algorithm a decode call with these tensors will use."""
+    a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
+                   None, None, algo, check_device=False)
+    if num_cus > 0:
+        a.flags |= _lib.FDK_FLAG_DRY_RUN
+    return _plan_of(a, num_cus)
+
+
+class PreparedDecode:
+    """A fully bound decode call: arguments marshalled once, ``run()`` only enqueues the kernels.
+
+    Keeps references to every tensor it points to.  ``run`` may be called repeatedly (e.g. from a
+    serving loop or while capturing a HIP graph): it allocates nothing and does not synchronise."""
+
+    def __init__(self, args: FdkDecodeArgs, plan: SplitKvPlan, keep: tuple, out, lse):
+        self.args = args
+        self.plan = plan
+        self._keep = keep
+        self.out = out
+        self.lse = lse
+        self._ref = C.byref(args)
+
+    def run(self, stream=None):
+        _lib.check(_LIB.fdk_decode(self._ref, _stream_handle(stream)))
+        return self.out, self.lse
+
+    def run_splitkv(self, stream=None):
+        _lib.check(_LIB.fdk_decode_splitkv(self._ref, _stream_handle(stream)))
+
+    def run_combine(self, stream=None):
+        _lib.check(_LIB.fdk_combine(self._ref, _stream_handle(stream)))
+        return self.out, self.lse
+
+
+def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
+                   max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
+                   algo="auto", packed_out=None, want_lse=True, always_workspace=False) -> PreparedDecode:
+    """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
+
+    ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
+    dtype) in ``[..., D]`` - the reference's ``output_combine`` layout - instead of ``out``."""
+    if not isinstance(kv_lens, torch.Tensor):
+        kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
+    a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
+                   k_scale, v_scale, algo)
+    batch, q_heads, d = q.shape
+    plan = _plan_of(a)
+    if packed_out is not None:
+        if tuple(packed_out.shape) != (batch, q_heads, d + 1) or packed_out.stride(-1) != 1:
+            raise ValueError(f"packed output must be [B, Hq, D+1] = {(batch, q_heads, d + 1)}")
+        a.flags |= _lib.FDK_FLAG_PACK_LSE
+        target = packed_out
+    else:
+        if out is None:
+            out = torch.empty((batch, q_heads, d), dtype=q.dtype, device=q.device)
+        elif tuple(out.shape) != (batch, q_heads, d) or out.stride(-1) != 1:
+            raise ValueError(f"out must be [B, Hq, D] = {(batch, q_heads, d)} with contiguous D")
+        target = out
+    if not target.is_cuda:
+        raise ValueError("output tensor must live on the GPU")
+    a.out = target.data_ptr()
+    a.out_stride_b, a.out_stride_h = target.stride(0), target.stride(1)
+    a.out_dtype = _fdk_dtype(target.dtype, "out")
+    if lse is None and want_lse:
+        lse = torch.empty((batch, q_heads), dtype=torch.float32, device=q.device)
+    if lse is not None:
+        if lse.dtype != torch.float32 or tuple(lse.shape) != (batch, q_heads) or lse.stride(-1) != 1:
+            raise ValueError("lse must be fp32 [B, Hq] with contiguous heads")
+        a.lse = lse.data_ptr()
+        a.lse_stride_b = lse.stride(0) if batch > 1 else max(lse.stride(0), q_heads)
+    need = plan.workspace_bytes if (plan.num_splits > 1 or always_workspace) else 0
+    if need:
+        if workspace is not None and (not workspace.is_cuda or not workspace.is_contiguous() or
+                                      workspace.numel() * workspace.element_size() < need or
+                                      workspace.data_ptr() % 16):
+            workspace = None        # too small / unusable: take our own
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        a.workspace = workspace.data_ptr()
+        a.workspace_bytes = workspace.numel() * workspace.element_size()
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace)
+    return PreparedDecode(a, plan, keep, target, lse)
+
+
+def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                 kv_lens: Union[torch.Tensor, Sequence[int]], sm_scale: float, *, soft_cap: float = 0.0,
+                 kv_split: int = -1, max_kv_len: Optional[int] = None, k_scale: Optional[torch.Tensor] = None,
+                 v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                 lse: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                 algo: str = "auto", stream=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Local (one GPU's share) split-KV GQA decode attention over a paged KV cache.
+
+    q            [B, Hq, D] bf16/fp16, one query token per sequence
+    k_cache      [num_pages, P, Hkv, D] in q's dtype or float8_e4m3fn
+    v_cache      same shape and dtype as k_cache
+    block_table  [B, max_pages] int32: page of token n is ``block_table[b, n // P]``, slot ``n % P``
+    kv_lens      [B] int32 (device tensor; never read on the host)
+    sm_scale     logit scale
+    soft_cap     > 0: logits become ``soft_cap * tanh(logits / soft_cap)``
+    kv_split     force this many KV splits (default: chosen from the shape and the CU count)
+    max_kv_len   host-known upper bound of kv_lens, used only to size the splits
+                 (default ``max_pages * P``)
+    k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
+
+    Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
+    and lse = ln sum exp(scaled logits) - what the cross-rank combine consumes."""
+    call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
+                          kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
+                          out=out, lse=lse, workspace=workspace, algo=algo)
+    return call.run(stream)
+
+
+def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                    soft_cap=0.0, output_split=None, output_combine=None, kv_split=-1,
+                                    stream=None):
+    """Drop-in for the reference function of the same name (flash_decode.py:847-928).
+
+    Returns ``output_combine [B, Hq, D+1]`` in q's dtype: attention output in ``[..., :D]``, lse in
+    ``[..., D]``.  ``workspace`` and ``q_lens`` are ignored as in the reference."""
+    batch, q_heads, d = q.shape
+    if output_combine is None:
+        output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
+    call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
+                          kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
+                          want_lse=False)
+    call.run(stream)
+    return output_combine
+
+
+def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
+                         output_split=None, output_combine=None, kv_split=-1, stream=None):
+    """Drop-in for the reference function of the same name (flash_decode.py:763-844): ``[B, Hq, D]``."""
+    call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
+                          kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
+                          want_lse=False)
+    return call.run(stream)[0]
+
+
+def gqa_fwd_batch_decode_intra_rank_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table,
+                                        scale, soft_cap=0, output_split=None, output_combine=None, kv_split=-1):
+    """Stream-first form (flash_decode.py:1037-1092)."""
+    return gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                           soft_cap, output_split, output_combine, kv_split, stream=stream)
+
+
+def gqa_fwd_batch_decode_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                             soft_cap=0, output_split=None, output_combine=None, kv_split=-1):
+    """Stream-first form (flash_decode.py:979-1034)."""
+    return gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap,
+                                output_split, output_combine, kv_split, stream=stream)
+
+
+def _as_scratch(output_split: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if output_split is None or not output_split.is_contiguous():
+        return None
+    return output_split.view(-1).view(torch.uint8)
+
+
+def pack_out_lse(out: torch.Tensor, lse: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``(out [B,Hq,D], lse [B,Hq]) -> [B,Hq,D+1]`` with lse in the last column (flash_decode.py:235-239)."""
+    dtype = dtype or out.dtype
+    packed = torch.empty(out.shape[:-1] + (out.shape[-1] + 1,), dtype=dtype, device=out.device)
+    packed[..., :-1] = out
+    packed[..., -1] = lse
+    return packed
+
+
+def unpack_out_lse(packed: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Inverse of ``pack_out_lse`` (views, no copy)."""
+    return packed[..., :-1], packed[..., -1]
+
+
+def inter_rank_combine(all_ranks_output: torch.Tensor, global_kv_lens: torch.Tensor,
+                       final_output: Optional[torch.Tensor] = None, *, all_ranks_lse: Optional[torch.Tensor] = None,
+                       lse_out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """Merge per-rank local results into the global attention output.
+
+    all_ranks_output  ``[R, B, Hq, D+1]`` packed (the all-gathered buffer of
+                      sp_flash_decode_layer.py:143-145) or ``[R, B, Hq, D]`` together with
+                      ``all_ranks_lse [R, B, Hq]`` fp32
+    global_kv_lens    ``[R, B]`` int32; rank r takes part for sequence b iff ``> 0`` (flash_decode.py:513-515)
+    Returns ``final_output [B, Hq, D]`` in the input dtype."""
+    if all_ranks_output.dim() != 4:
+        raise ValueError("all_ranks_output must be [R, B, Hq, D(+1)]")
+    n_ranks, batch, q_heads, last = all_ranks_output.shape
+    packed = all_ranks_lse is None
+    d = last - 1 if packed else last
+    if all_ranks_output.stride(-1) != 1:
+        raise ValueError("last dimension must be contiguous")
+    if global_kv_lens.dtype != torch.int32 or tuple(global_kv_lens.shape) != (n_ranks, batch) or \
+            not global_kv_lens.is_contiguous():
+        raise ValueError("global_kv_lens must be contiguous int32 [R, B]")
+    if not all_ranks_output.is_cuda or not global_kv_lens.is_cuda:
+        raise ValueError("inputs must live on the GPU; there is no CPU path")
+    if final_output is None:
+        final_output = torch.empty((batch, q_heads, d), dtype=all_ranks_output.dtype, device=all_ranks_output.device)
+    a = FdkCombineRanksArgs()
+    a.struct_size = C.sizeof(FdkCombineRanksArgs)
+    a.flags = _lib.FDK_FLAG_PACK_LSE if packed else 0
+    a.partial = all_ranks_output.data_ptr()
+    a.stride_r, a.stride_b, a.stride_h = all_ranks_output.stride(0), all_ranks_output.stride(1), all_ranks_output.stride(2)
+    a.partial_dtype = _fdk_dtype(all_ranks_output.dtype, "all_ranks_output")
+    a.out_dtype = _fdk_dtype(final_output.dtype, "final_output")
+    if not packed:
+        if all_ranks_lse.dtype != torch.float32 or tuple(all_ranks_lse.shape) != (n_ranks, batch, q_heads) or \
+                all_ranks_lse.stride(-1) != 1:
+            raise ValueError("all_ranks_lse must be fp32 [R, B, Hq]")
+        a.partial_lse = all_ranks_lse.data_ptr()
+        a.lse_stride_r, a.lse_stride_b = all_ranks_lse.stride(0), all_ranks_lse.stride(1)
+    a.kv_lens = global_kv_lens.data_ptr()
+    a.num_ranks, a.batch, a.num_q_heads, a.head_dim = n_ranks, batch, q_heads, d
+    a.out = final_output.data_ptr()
+    a.out_stride_b, a.out_stride_h = final_output.stride(0), final_output.stride(1)
+    if lse_out is not None:
+        a.lse = lse_out.data_ptr()
+        a.lse_stride_b_out = lse_out.stride(0)
+    _lib.check(_LIB.fdk_combine_ranks(C.byref(a), _stream_handle(stream)))
+    return final_output
