@@ -290,10 +290,10 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
     g = torch.Generator().manual_seed(13)
     shard_lens = torch.tensor([[512, 16, 0], [300, 0, 0], [0, 77, 0], [1, 1000, 5]], dtype=torch.int32)
     q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
-    pool = 80
+    pool = 200
     ks = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
     vs = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
-    tables = [torch.randperm(pool, generator=g)[:b * 21].view(b, 21).to(torch.int32).to(cuda_device) for _ in range(r_)]
+    tables = [torch.randperm(pool, generator=g)[:b * 63].view(b, 63).to(torch.int32).to(cuda_device) for _ in range(r_)]
     packed = torch.full((r_, b, hq, d + 1), float("nan"), dtype=torch.float32, device=cuda_device)
     outs = torch.empty(r_, b, hq, d, dtype=torch.bfloat16, device=cuda_device)
     lses = torch.empty(r_, b, hq, dtype=torch.float32, device=cuda_device)
@@ -326,7 +326,7 @@ def test_page_sizes_that_are_not_powers_of_two(cuda_device, page):
     if c is None:
         g = torch.Generator().manual_seed(41)
         lens = [500, 23, 24, 25]
-        pool = 60
+        pool = 100
         c = dict(q=torch.randn(4, 8, 128, generator=g).to(torch.bfloat16).to(cuda_device),
                  k_cache=torch.randn(pool, page, 2, 128, generator=g).to(torch.bfloat16).to(cuda_device),
                  v_cache=torch.randn(pool, page, 2, 128, generator=g).to(torch.bfloat16).to(cuda_device),
@@ -352,11 +352,12 @@ def test_fp8_kv_cache_small(cuda_device, heads):
     vd = ofp8.dequant_per_head(inp.v_cache, inp.v_scale)
     _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
            ref_kv=(kd, vd), tag="fp8")
-    # and, tighter, the exact dequantisation in float64 (no bf16 rounding of the scaled values)
+    # the exact dequantisation in float64 (no bf16 rounding of k8*scale) is a different function of the bytes:
+    # rounding K to bf16 moves single logits by ~2^-9 relative, i.e. lse by up to a few 1e-3
     o64, l64 = cf.attn_fp64(inp.q, inp.k_cache.float(), inp.v_cache.float(), inp.block_table, inp.kv_lens_host,
                             inp.sm_scale, k_scale=inp.k_scale, v_scale=inp.v_scale)
     torch.testing.assert_close(out.double(), o64, atol=5e-3, rtol=1e-2)
-    torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0)
+    torch.testing.assert_close(lse.double(), l64, atol=5e-3, rtol=0)
 
 
 def test_fp8_every_byte_value_dequantises_exactly(cuda_device):

@@ -212,6 +212,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.group = a->num_q_heads / a->num_kv_heads;
     sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
     sp.num_splits = S; sp.chunk = r->plan.chunk_tokens;
+    sp.max_tokens = (int32_t)((int64_t)a->max_pages * a->page_size);
     sp.head_tiles = r->plan.reserved;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
@@ -227,6 +228,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     cp.out_sb = a->out_stride_b; cp.out_sh = a->out_stride_h; cp.lse_sb = a->lse_stride_b;
     cp.batch = a->batch; cp.hq = a->num_q_heads;
     cp.num_splits = S; cp.chunk = r->plan.chunk_tokens;
+    cp.max_tokens = sp.max_tokens;
     cp.out_dtype = a->out_dtype; cp.pack_lse = sp.pack_lse;
     return FDK_OK;
 }

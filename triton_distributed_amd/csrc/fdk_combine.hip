@@ -22,7 +22,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + wave;   // b * Hq + h
     if (row >= (int64_t)p.batch * p.hq) return;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
-    const int kv_len = p.kv_lens[b];
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
     // live splits: chunk c holds tokens [c*chunk, ...) - the split kernel wrote exactly these
     const int live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
 

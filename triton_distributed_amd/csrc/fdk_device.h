@@ -35,6 +35,7 @@ struct SplitParams {
     int32_t batch, hq, hkv, group;
     int32_t page_size, page_shift;  // page_shift = log2(page_size) or -1
     int32_t num_splits, chunk;
+    int32_t max_tokens;             // block_table columns * page_size: kv_len is clamped to it
     int32_t head_tiles;             // ceil(group / heads-per-workgroup)
     int32_t out_dtype;              // fdk_dtype
     int32_t pack_lse;
@@ -53,6 +54,7 @@ struct CombineParams {
     int64_t out_sb, out_sh, lse_sb;
     int32_t batch, hq;
     int32_t num_splits, chunk;
+    int32_t max_tokens;
     int32_t out_dtype;
     int32_t pack_lse;
 };
@@ -137,12 +139,6 @@ template <> struct Pack2<FDK_BF16> {
         vec r = {(__bf16)a, (__bf16)b};
         return __builtin_bit_cast(uint32_t, r);
     }
-    static __device__ __forceinline__ uint32_t from_fp8_lo(uint32_t w) {  // bytes 0,1 -> two bf16
-        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
-    }
-    static __device__ __forceinline__ uint32_t from_fp8_hi(uint32_t w) {  // bytes 2,3
-        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
-    }
 };
 template <> struct Pack2<FDK_FP16> {
     using vec = f16x2_t;
@@ -154,12 +150,6 @@ template <> struct Pack2<FDK_FP16> {
     static __device__ __forceinline__ uint32_t pack(float a, float b) {
         vec r = {(_Float16)a, (_Float16)b};
         return __builtin_bit_cast(uint32_t, r);
-    }
-    static __device__ __forceinline__ uint32_t from_fp8_lo(uint32_t w) {
-        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
-    }
-    static __device__ __forceinline__ uint32_t from_fp8_hi(uint32_t w) {
-        return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
     }
 };
 

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void splitkv_valu_kernel(const SplitParams p) 
     const int head0 = kvh * p.group + ht * GT;       // first q head of this workgroup
     const int heads_here = min(GT, p.group - ht * GT);
 
-    const int kv_len = p.kv_lens[b];
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
     const int c_start = split * p.chunk;
     if (c_start >= kv_len) {
         if (p.direct) {   // kv_len == 0 with a single split: defined result, no combine follows
@@ -117,8 +117,8 @@ __global__ __launch_bounds__(256) void splitkv_valu_kernel(const SplitParams p) 
         if (p.k_scale) kscale = p.k_scale[kvh];
         if (p.v_scale) vscale = p.v_scale[kvh];
     }
-    const float scale_log2 = p.scale_log2 * kscale;      // raw dot -> log2-unit logit
-    const float scale_nat = p.sm_scale * kscale;          // raw dot -> natural-unit logit (soft cap)
+    const float scale_log2 = p.scale_log2;               // raw dot -> log2-unit logit
+    const float scale_nat = p.sm_scale;                   // raw dot -> natural-unit logit (soft cap)
     const bool softcap = p.soft_cap > 0.f;
     const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
 
@@ -192,10 +192,14 @@ __global__ __launch_bounds__(256) void splitkv_valu_kernel(const SplitParams p) 
         for (int j = 0; j < NJ; ++j) {
             uint32_t kk[QW];
             if (FP8) {
+                // dequantise exactly as "(k8 * scale) rounded to the q dtype": the logits, and with them
+                // lse, then equal those of a decode over the dequantised cache
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    kk[2 * w] = P2::from_fp8_lo(kt.k[j][w]);
-                    kk[2 * w + 1] = P2::from_fp8_hi(kt.k[j][w]);
+                    const f32x2_t f01 = __builtin_amdgcn_cvt_pk_f32_fp8(kt.k[j][w], false);
+                    const f32x2_t f23 = __builtin_amdgcn_cvt_pk_f32_fp8(kt.k[j][w], true);
+                    kk[2 * w] = P2::pack(f01.x * kscale, f01.y * kscale);
+                    kk[2 * w + 1] = P2::pack(f23.x * kscale, f23.y * kscale);
                 }
             } else {
 #pragma unroll
