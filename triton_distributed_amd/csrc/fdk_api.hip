@@ -143,7 +143,11 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
 
     const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group) : fdk::valu_heads_per_wg(group);
     const int head_tiles = (group + hpw - 1) / hpw;
-    const int64_t units = (int64_t)(a->batch > 0 ? a->batch : 1) * a->num_kv_heads * head_tiles;
+    const bool heads_contiguous = a->k_stride_head == fdk::kHeadDim && a->v_stride_head == fdk::kHeadDim;
+    const int units_per_seq = algo == FDK_ALGO_MFMA
+                                  ? a->num_kv_heads * head_tiles
+                                  : fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
+    const int64_t units = (int64_t)(a->batch > 0 ? a->batch : 1) * units_per_seq;
 
     int64_t splits;
     if (a->num_splits > 0) {
@@ -170,6 +174,12 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     return FDK_OK;
 }
 
+int head_tiles_of(const fdk_decode_args* a) {
+    const int group = a->num_q_heads / a->num_kv_heads;
+    const int hpw = fdk::valu_heads_per_wg(group);
+    return (group + hpw - 1) / hpw;
+}
+
 struct Resolved {
     fdk_plan_t plan;
     fdk::SplitParams sp;
@@ -182,7 +192,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     const int S = r->plan.num_splits;
     const bool direct = direct_ok && S == 1;
     const int64_t rows = (int64_t)a->batch * a->num_q_heads;
-    if ((int64_t)a->batch * S * a->num_kv_heads * r->plan.reserved > INT32_MAX)
+    if ((int64_t)a->batch * S * a->num_kv_heads * head_tiles_of(a) > INT32_MAX)
         return fail(FDK_ESHAPE, "grid too large");
     float* part_o = nullptr;
     float* part_lse = nullptr;

@@ -37,6 +37,7 @@ struct SplitParams {
     int32_t num_splits, chunk;
     int32_t max_tokens;             // block_table columns * page_size: kv_len is clamped to it
     int32_t head_tiles;             // ceil(group / heads-per-workgroup)
+    int32_t hg_per_wg, hg_blocks;   // kv-head groups per workgroup / workgroups along the kv-head axis
     int32_t out_dtype;              // fdk_dtype
     int32_t pack_lse;
     int32_t direct;                 // 1: single split, write the final (out, lse) instead of partials
@@ -78,6 +79,8 @@ int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStre
 int launch_combine(const CombineParams& p, hipStream_t stream);
 int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
 bool valu_supported(int q_dtype, int kv_dtype, int group);
+// workgroups per (sequence, split) of the VALU path for this head layout
+int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
 bool mfma_supported(int q_dtype, int kv_dtype, int group);
 int valu_heads_per_wg(int group);
 int mfma_heads_per_wg(int group);
