@@ -57,8 +57,9 @@ def _check(out, lse, q, k, v, table, lens, scale, soft_cap=0.0, k_scale=None, v_
 @pytest.mark.parametrize("block_size", [1, 16])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("soft_cap", [0, 30, 50])
-def test_reference_grid(cuda_device, kv_lens, num_heads, block_size, dtype, soft_cap):
-    print(f"case lens={kv_lens} heads={num_heads} P={block_size} {dtype} cap={soft_cap}", flush=True)
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_reference_grid(cuda_device, kv_lens, num_heads, block_size, dtype, soft_cap, algo):
+    print(f"case lens={kv_lens} heads={num_heads} P={block_size} {dtype} cap={soft_cap} {algo}", flush=True)
     num_blocks = 1024
     g = torch.Generator(device="cpu").manual_seed(hash((tuple(kv_lens), num_heads, block_size, soft_cap)) & 0xFFFF)
     hq, hkv = num_heads
@@ -70,9 +71,11 @@ def test_reference_grid(cuda_device, kv_lens, num_heads, block_size, dtype, soft
     max_blocks = (max(kv_lens) + block_size - 1) // block_size
     table = torch.randint(0, num_blocks, (len(kv_lens), max_blocks), generator=g, dtype=torch.int32).to(cuda_device)
     lens_t = _lens_t(kv_lens, cuda_device)
-    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap))
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap), algo=algo)
     torch.cuda.synchronize()
     _check(out, lse, q, k, v, table, kv_lens, scale, float(soft_cap), tag="grid")
+    if algo != tda.get_split_kv_plan(q, k, v, table, lens_t).algo:
+        return                                      # the reference-named entry points use the default algorithm
     # the reference entry points: same numbers, reference layouts
     o2 = tda.gqa_fwd_batch_decode(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale, float(soft_cap))
     packed = tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale,
@@ -112,12 +115,13 @@ def test_head_dim_256_is_rejected(cuda_device):
 # ---- golden vectors and edge cases -----------------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["tiny", *EDGE_CASES])
 @pytest.mark.parametrize("kv_split", [-1, 1, 3, 32])
-def test_golden_cases(cuda_device, name, kv_split):
-    print(f"case golden {name} kv_split={kv_split}", flush=True)
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_golden_cases(cuda_device, name, kv_split, algo):
+    print(f"case golden {name} kv_split={kv_split} {algo}", flush=True)
     c = _dev(dict(all_cases())[name], cuda_device)
     lens_t = _lens_t(c["kv_lens"], cuda_device)
     out, lse = tda.flash_decode(c["q"], c["k_cache"], c["v_cache"], c["block_table"], lens_t, c["sm_scale"],
-                                soft_cap=c["soft_cap"], kv_split=kv_split)
+                                soft_cap=c["soft_cap"], kv_split=kv_split, algo=algo)
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
     np.testing.assert_allclose(out.float().cpu().numpy(), GOLDEN[name + ".ref"], atol=OUT_ATOL, rtol=OUT_RTOL)
@@ -126,7 +130,8 @@ def test_golden_cases(cuda_device, name, kv_split):
 
 
 @pytest.mark.parametrize("page", [1, 16])
-def test_single_token_sequences_are_bit_exact_gathers(cuda_device, page):
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_single_token_sequences_are_bit_exact_gathers(cuda_device, page, algo):
     g = torch.Generator().manual_seed(31)
     b, hq, hkv, d, pool = 7, 8, 2, 128, 50
     q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
@@ -134,7 +139,7 @@ def test_single_token_sequences_are_bit_exact_gathers(cuda_device, page):
     v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
     table = torch.randint(0, pool, (b, 3), generator=g, dtype=torch.int32).to(cuda_device)
     table[:, 1:] = 2**31 - 1                                       # never read
-    out, lse = tda.flash_decode(q, k, v, table, _lens_t([1] * b, cuda_device), d ** -0.5)
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t([1] * b, cuda_device), d ** -0.5, algo=algo)
     torch.cuda.synchronize()
     for i in range(b):
         for h in range(hq):
@@ -207,7 +212,8 @@ def test_poisoned_table_tail_is_never_read(cuda_device):
 
 
 @pytest.mark.parametrize("kv_split", [32, 64])
-def test_short_sequences_and_empty_splits_stay_finite(cuda_device, kv_split):
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_short_sequences_and_empty_splits_stay_finite(cuda_device, kv_split, algo):
     lens = [1, 2, kv_split - 1, kv_split, kv_split + 1, 63, 64, 65, 255, 256, 257]
     g = torch.Generator().manual_seed(77)
     hq, hkv, d, page = 8, 2, 128, 16
@@ -223,7 +229,7 @@ def test_short_sequences_and_empty_splits_stay_finite(cuda_device, kv_split):
             k[last, n % page:] = float("nan")
             v[last, n % page:] = float("nan")
     # force real splitting of short sequences: pretend the host bound is the table width
-    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5, kv_split=kv_split)
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5, kv_split=kv_split, algo=algo)
     torch.cuda.synchronize()
     kc, vc = torch.nan_to_num(k), torch.nan_to_num(v)
     _check(out, lse, q, kc, vc, table, lens, d ** -0.5, tag=f"short S={kv_split}")
@@ -321,7 +327,8 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
 
 
 @pytest.mark.parametrize("page", [6, 24])
-def test_page_sizes_that_are_not_powers_of_two(cuda_device, page):
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_page_sizes_that_are_not_powers_of_two(cuda_device, page, algo):
     c = _dev(dict(all_cases())["odd_page6"], cuda_device) if page == 6 else None
     if c is None:
         g = torch.Generator().manual_seed(41)
@@ -333,19 +340,20 @@ def test_page_sizes_that_are_not_powers_of_two(cuda_device, page):
                  block_table=torch.randperm(pool, generator=g)[:4 * 21].view(4, 21).to(torch.int32).to(cuda_device),
                  kv_lens=lens, sm_scale=128 ** -0.5, soft_cap=0.0)
     out, lse = tda.flash_decode(c["q"], c["k_cache"], c["v_cache"], c["block_table"], _lens_t(c["kv_lens"], cuda_device),
-                                c["sm_scale"])
+                                c["sm_scale"], algo=algo)
     torch.cuda.synchronize()
     _check(out, lse, c["q"], c["k_cache"], c["v_cache"], c["block_table"], c["kv_lens"], c["sm_scale"], tag=f"P={page}")
 
 
 # ---- fp8 KV cache ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("heads", [(32, 8), (64, 8), (8, 8)])
-def test_fp8_kv_cache_small(cuda_device, heads):
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_fp8_kv_cache_small(cuda_device, heads, algo):
     cfg = wl.DecodeConfig("fp8_small", 55, 5, heads[0], heads[1], 128, 16, kv_len_range=(1, 2000), kv_dtype="fp8_e4m3",
                           spare_pages=4)
     inp = wl.make_inputs(cfg, cuda_device, poison_tail=True)
     out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
-                                k_scale=inp.k_scale, v_scale=inp.v_scale)
+                                k_scale=inp.k_scale, v_scale=inp.v_scale, algo=algo)
     torch.cuda.synchronize()
     # the workload's definition: dequantise to bf16, then the same decode
     kd = ofp8.dequant_per_head(inp.k_cache, inp.k_scale)
@@ -360,7 +368,8 @@ def test_fp8_kv_cache_small(cuda_device, heads):
     torch.testing.assert_close(lse.double(), l64, atol=5e-3, rtol=0)
 
 
-def test_fp8_every_byte_value_dequantises_exactly(cuda_device):
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_fp8_every_byte_value_dequantises_exactly(cuda_device, algo):
     # 254 finite e4m3 codes as single-token V rows: out must equal table[code] * scale bit-exactly in fp32
     table = torch.from_numpy(ofp8.e4m3fn_table())
     codes = torch.tensor([c for c in range(256) if not math.isnan(table[c])], dtype=torch.uint8)
@@ -371,19 +380,25 @@ def test_fp8_every_byte_value_dequantises_exactly(cuda_device):
     scale = torch.tensor([0.75], device=cuda_device)
     bt = torch.arange(n, dtype=torch.int32, device=cuda_device)[:, None].contiguous()
     out = torch.empty(n, 1, 128, dtype=torch.float32, device=cuda_device)
-    tda.flash_decode(q, k8, v8, bt, _lens_t([1] * n, cuda_device), 1.0, k_scale=scale, v_scale=scale, out=out)
+    tda.flash_decode(q, k8, v8, bt, _lens_t([1] * n, cuda_device), 1.0, k_scale=scale, v_scale=scale, out=out, algo=algo)
     torch.cuda.synchronize()
     want = (table[codes.long()] * 0.75).to(cuda_device)
     assert torch.equal(out[:, 0, 0], want) and torch.equal(out[:, 0, 127], want)
 
 
 # ---- the five benchmark configurations at full size ----------------------------------------------------------------
-def _full_config(name, cuda_device, lse_rows=None):
-    print(f"config {name}: generating", flush=True)
-    inp = wl.make_inputs(name, cuda_device)
-    print(f"config {name}: decode", flush=True)
+_INPUT_CACHE = {}
+
+
+def _full_config(name, cuda_device, algo="auto"):
+    if name not in _INPUT_CACHE:
+        _INPUT_CACHE.clear()                         # one configuration resident at a time
+        print(f"config {name}: generating", flush=True)
+        _INPUT_CACHE[name] = wl.make_inputs(name, cuda_device)
+    inp = _INPUT_CACHE[name]
+    print(f"config {name}: decode ({algo})", flush=True)
     out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
-                                k_scale=inp.k_scale, v_scale=inp.v_scale)
+                                k_scale=inp.k_scale, v_scale=inp.v_scale, algo=algo)
     torch.cuda.synchronize()
     assert out.shape == inp.q.shape and out.dtype == torch.bfloat16 and lse.dtype == torch.float32
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
@@ -408,29 +423,32 @@ def _check_rows(inp, out, lse, rows, tag):
             _check(out[sl], lse[sl], inp.q[sl], k, v, inp.block_table[sl], lens, inp.sm_scale, tag=f"{tag} b={b}")
 
 
-def test_config1_tiny(cuda_device):
-    inp, out, lse = _full_config("tiny", cuda_device)
+@pytest.mark.parametrize("algo", ["auto", "valu", "mfma"])
+def test_config1_tiny(cuda_device, algo):
+    inp, out, lse = _full_config("tiny", cuda_device, algo)
     assert out.shape == (2, 8, 128) and lse.shape == (2, 8)
     _check_rows(inp, out, lse, range(2), "tiny")
 
 
-def test_config2_llama3_8b_b32(cuda_device):
-    inp, out, lse = _full_config("llama3_8b_b32", cuda_device)
-    _check_rows(inp, out, lse, range(32), "cfg2")
+@pytest.mark.parametrize("algo", ["auto", "valu", "mfma"])
+def test_config2_llama3_8b_b32(cuda_device, algo):
+    inp, out, lse = _full_config("llama3_8b_b32", cuda_device, algo)
+    _check_rows(inp, out, lse, range(32) if algo == "auto" else range(0, 32, 5), "cfg2")
 
 
-def test_config3_ragged_g8(cuda_device):
-    inp, out, lse = _full_config("ragged_g8", cuda_device)
-    _check_rows(inp, out, lse, range(64), "cfg3")
+@pytest.mark.parametrize("algo", ["auto", "valu"])
+def test_config3_ragged_g8(cuda_device, algo):
+    inp, out, lse = _full_config("ragged_g8", cuda_device, algo)
+    _check_rows(inp, out, lse, range(64) if algo == "auto" else range(0, 64, 7), "cfg3")
 
 
-def test_config4_long_131k(cuda_device):
-    inp, out, lse = _full_config("long_131k", cuda_device)
-    _check_rows(inp, out, lse, range(4), "cfg4")
+@pytest.mark.parametrize("algo", ["auto", "valu"])
+def test_config4_long_131k(cuda_device, algo):
+    inp, out, lse = _full_config("long_131k", cuda_device, algo)
+    _check_rows(inp, out, lse, range(4) if algo == "auto" else [3], "cfg4")
 
 
-def test_config5_fp8_70b_b128(cuda_device):
-    inp, out, lse = _full_config("fp8_70b_b128", cuda_device)
-    _check_rows(inp, out, lse, range(0, 128, 9), "cfg5")
-    # size-independent property at full size: the same sequence placed twice gives the same rows
-    assert torch.isfinite(out.float()).all()
+@pytest.mark.parametrize("algo", ["auto", "valu"])
+def test_config5_fp8_70b_b128(cuda_device, algo):
+    inp, out, lse = _full_config("fp8_70b_b128", cuda_device, algo)
+    _check_rows(inp, out, lse, range(0, 128, 9) if algo == "auto" else [5, 100], "cfg5")
