@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--kv-split", type=int, default=-1)
     ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
+                         "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
     return ap.parse_args()
 
@@ -138,6 +141,14 @@ def main():
     torch.cuda.synchronize()
     if not (torch.isfinite(out.float()).all() and torch.isfinite(lse).all()):
         raise RuntimeError("non-finite decode output on the benchmark inputs")
+
+    if args.copy_calibration > 0:
+        src = torch.full((args.copy_calibration << 20,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def step(i):
         calls[i % len(calls)].run()

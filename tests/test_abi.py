@@ -115,8 +115,6 @@ def test_valid_arguments_pass_dry_run():
     ("kv_dtype", _lib.FDK_FP16, _lib.FDK_EUNSUPPORTED),
     ("out_dtype", _lib.FDK_FP8_E4M3, _lib.FDK_EUNSUPPORTED),
     ("algo", 7, _lib.FDK_EUNSUPPORTED),
-    ("workspace", None, _lib.FDK_EWORKSPACE),
-    ("workspace_bytes", 1024, _lib.FDK_EWORKSPACE),
     ("sm_scale", float("nan"), _lib.FDK_ESHAPE),
 ])
 def test_bad_arguments_are_rejected_without_a_launch(field, value, code):
@@ -125,6 +123,17 @@ def test_bad_arguments_are_rejected_without_a_launch(field, value, code):
     assert len(_lib.load().fdk_last_error()) > 0
     with pytest.raises((ValueError, _lib.FdkError)):
         _lib.check(rc)
+
+
+def test_workspace_is_required_only_when_the_plan_splits():
+    # 32 sequences x 8 kv heads fill 256 compute units on their own: one pass, no scratch
+    assert _decode_rc(_args(workspace=None, workspace_bytes=0)) == 0
+    # 4 sequences do not: the KV range is split and the partials need scratch
+    assert _decode_rc(_args(batch=4, workspace=None)) == _lib.FDK_EWORKSPACE
+    assert _decode_rc(_args(batch=4, workspace_bytes=1024)) == _lib.FDK_EWORKSPACE
+    assert _decode_rc(_args(batch=4)) == 0
+    # a forced split count needs it as well
+    assert _decode_rc(_args(num_splits=4, workspace=None)) == _lib.FDK_EWORKSPACE
 
 
 def test_packed_output_needs_a_wider_row():
@@ -150,28 +159,30 @@ def _plan(a, cus=256):
 
 
 def test_plan_scales_splits_with_occupancy():
-    p = _plan(_args())                                    # 256 (b, kv head) units on 256 CUs
-    assert p.num_splits >= 2 and p.chunk_tokens % 64 == 0
-    assert p.num_splits * p.chunk_tokens >= 4096 > (p.num_splits - 1) * p.chunk_tokens
-    assert p.algo == _lib.FDK_ALGO_VALU                   # group 4: vector path
+    p = _plan(_args())                                    # 256 (sequence, kv head) units on 256 CUs
+    assert p.num_splits == 1 and p.chunk_tokens >= 4096   # they fill the device: one pass, no combine
+    assert p.algo == _lib.FDK_ALGO_MFMA
+    # fewer sequences: the KV range is split, chunks are multiples of 64 tokens and cover the range
+    p4 = _plan(_args(batch=4))
+    assert p4.num_splits > 1 and p4.chunk_tokens % 64 == 0
+    assert p4.num_splits * p4.chunk_tokens >= 4096 > (p4.num_splits - 1) * p4.chunk_tokens
     # few units, long context -> many splits; chunks never shorter than 256 tokens
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
                          q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
-    assert p_long.num_splits > p.num_splits and p_long.chunk_tokens >= 256
-    # huge batch -> no split at all
-    p_big = _plan(_args(batch=4096))
-    assert p_big.num_splits == 1
+    assert p_long.num_splits > p4.num_splits and p_long.chunk_tokens >= 512
     # short context is never split below the minimum chunk
     p_short = _plan(_args(batch=1, max_pages=8, table_stride_b=8))
     assert p_short.num_splits == 1 and p_short.chunk_tokens >= 128
     # the host's bound on kv_len drives the split, not the table width
-    p_hint = _plan(_args(max_pages=2048, table_stride_b=2048, max_kv_len=4096))
-    assert (p_hint.num_splits, p_hint.chunk_tokens) == (p.num_splits, p.chunk_tokens)
+    p_hint = _plan(_args(batch=4, max_pages=2048, table_stride_b=2048, max_kv_len=4096))
+    assert (p_hint.num_splits, p_hint.chunk_tokens) == (p4.num_splits, p4.chunk_tokens)
     # a forced split count is honoured and covers the whole range
     p_forced = _plan(_args(num_splits=32))
     assert p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
-    # fewer compute units -> fewer splits
-    assert _plan(_args(), cus=64).num_splits <= p.num_splits
+    # fewer compute units -> no more splits than with many
+    assert _plan(_args(batch=4), cus=64).num_splits <= p4.num_splits
+    # the vector path can be forced
+    assert _plan(_args(algo=_lib.FDK_ALGO_VALU)).algo == _lib.FDK_ALGO_VALU
 
 
 def test_workspace_bytes_formula():

@@ -48,7 +48,7 @@ def test_shape_and_dtype_checks_mirror_the_reference_asserts():
 def test_plan_from_tensors():
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=2, kv_len=4096))
     p = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, num_cus=256)
-    assert p.algo == "valu" and p.num_splits * p.chunk_tokens >= 4096 and p.workspace_bytes > 0
+    assert p.algo == "mfma" and p.num_splits * p.chunk_tokens >= 4096 and p.workspace_bytes > 0
     p32 = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, kv_split=32, num_cus=256)
     assert p32.num_splits == 32
 

@@ -58,7 +58,7 @@ int query_cus() {
 }
 
 constexpr int kChunkAlign = 64;     // split boundaries fall on multiples of 64 tokens
-constexpr int kMinChunk = 256;      // never split finer than this
+constexpr int kMinChunk = 512;      // never split finer than this
 constexpr int kMaxSplits = 1024;
 
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
@@ -127,8 +127,9 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const int group = a->num_q_heads / a->num_kv_heads;
     int algo = a->algo;
     if (algo == FDK_ALGO_AUTO) {
-        // Matrix cores only where the q-head group makes a real tile (>= 8 heads per kv head).
-        algo = (group >= 8 && fdk::mfma_supported(a->q_dtype, a->kv_dtype, group)) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
+        // The matrix-core path is the default for every group size: on MI355X it is at least as fast as the
+        // vector path even for small groups, because it needs an order of magnitude fewer issue slots per KV byte.
+        algo = fdk::mfma_supported(a->q_dtype, a->kv_dtype, group) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
     }
     if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group))
         return fail(FDK_EUNSUPPORTED, "MFMA path not built for q_dtype=%d kv_dtype=%d group=%d", a->q_dtype,
@@ -141,22 +142,29 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     if (max_len > table_cap) max_len = table_cap;
     if (max_len < 1) max_len = 1;
 
-    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group) : fdk::valu_heads_per_wg(group);
-    const int head_tiles = (group + hpw - 1) / hpw;
+    if (num_cus <= 0) num_cus = query_cus();
+    const int batch = a->batch > 0 ? a->batch : 1;
     const bool heads_contiguous = a->k_stride_head == fdk::kHeadDim && a->v_stride_head == fdk::kHeadDim;
-    const int units_per_seq = algo == FDK_ALGO_MFMA
-                                  ? a->num_kv_heads * head_tiles
-                                  : fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
-    const int64_t units = (int64_t)(a->batch > 0 ? a->batch : 1) * units_per_seq;
+    int kv_heads_per_wg = 1;
+    int units_per_seq;
+    if (algo == FDK_ALGO_MFMA) {
+        kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus);
+        units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg);
+    } else {
+        units_per_seq = fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
+    }
+    const int64_t units = (int64_t)batch * units_per_seq;
 
+    // Split count: none when the (sequence, head block) units alone fill the compute units - a single pass
+    // then writes the final result and no combine runs.  Otherwise aim at two workgroups per compute unit,
+    // with chunks of at least kMinChunk tokens.
     int64_t splits;
     if (a->num_splits > 0) {
         splits = a->num_splits;
+    } else if (units >= num_cus) {
+        splits = 1;
     } else {
-        if (num_cus <= 0) num_cus = query_cus();
-        // Aim at ~8 workgroups (32 wavefronts) per compute unit, but keep chunks >= kMinChunk tokens.
-        const int64_t target = (int64_t)num_cus * 8;
-        splits = cdiv64(target, units);
+        splits = cdiv64(2 * (int64_t)num_cus, units);
         const int64_t cap = cdiv64(max_len, kMinChunk);
         if (splits > cap) splits = cap;
         if (splits < 1) splits = 1;
@@ -170,7 +178,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     plan->num_splits = (int32_t)splits;
     plan->chunk_tokens = (int32_t)chunk;
     plan->algo = algo;
-    plan->reserved = head_tiles;
+    plan->reserved = kv_heads_per_wg;
     return FDK_OK;
 }
 
@@ -223,7 +231,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
     sp.num_splits = S; sp.chunk = r->plan.chunk_tokens;
     sp.max_tokens = (int32_t)((int64_t)a->max_pages * a->page_size);
-    sp.head_tiles = r->plan.reserved;
+    sp.head_tiles = head_tiles_of(a);
+    sp.hg_per_wg = r->plan.reserved;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;

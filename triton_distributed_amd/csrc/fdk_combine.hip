@@ -66,6 +66,59 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     }
 }
 
+// Many splits: one workgroup per (sequence, head) row.  Every wavefront finds the global maximum and the sum
+// of weights (a few lse loads), then the four wavefronts share the partial rows (s = wave, wave+4, ...) with
+// eight independent loads in flight each, and the four sums meet in LDS.  Same result as combine_kernel.
+__global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p) {
+    __shared__ float sm[kRowsPerWg][kHeadDim];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t row = blockIdx.x;
+    const int b = (int)(row / p.hq), h = (int)(row % p.hq);
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
+    const int live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
+    const float* lse_row = p.part_lse + row * p.num_splits;
+    const float* o_row = p.part_o + row * p.num_splits * kHeadDim;
+
+    float m = -INFINITY;
+    for (int s0 = 0; s0 < live; s0 += 64) {
+        const float my = s0 + lane < live ? lse_row[s0 + lane] : -INFINITY;
+        m = fmaxf(m, wave_max(my));
+    }
+    m *= kLog2e;
+    float l = 0.f, acc0 = 0.f, acc1 = 0.f;
+    for (int s0 = 0; s0 < live; s0 += 64) {
+        const int n = min(64, live - s0);
+        const float w = lane < n ? fast_exp2(lse_row[s0 + lane] * kLog2e - m) : 0.f;
+        l += wave_sum(w);
+#pragma unroll 8
+        for (int s = wave; s < n; s += kRowsPerWg) {
+            const float ws = __shfl(w, s, 64);
+            const float2 o = *reinterpret_cast<const float2*>(o_row + (int64_t)(s0 + s) * kHeadDim + 2 * lane);
+            acc0 += ws * o.x;
+            acc1 += ws * o.y;
+        }
+    }
+    sm[wave][2 * lane] = acc0;
+    sm[wave][2 * lane + 1] = acc1;
+    __syncthreads();
+    if (wave != 0) return;
+    float r0 = 0.f, r1 = 0.f, lse = -INFINITY;
+    if (live > 0) {
+        const float inv = 1.0f / l;
+        r0 = (sm[0][2 * lane] + sm[1][2 * lane] + sm[2][2 * lane] + sm[3][2 * lane]) * inv;
+        r1 = (sm[0][2 * lane + 1] + sm[1][2 * lane + 1] + sm[2][2 * lane + 1] + sm[3][2 * lane + 1]) * inv;
+        lse = (m + fast_log2(l)) * kLn2;
+    }
+    const int64_t ob = (int64_t)b * p.out_sb + (int64_t)h * p.out_sh;
+    store_out(p.out, ob + 2 * lane, r0, p.out_dtype);
+    store_out(p.out, ob + 2 * lane + 1, r1, p.out_dtype);
+    if (lane == 0) {
+        if (p.lse) p.lse[(int64_t)b * p.lse_sb + h] = lse;
+        if (p.pack_lse) store_out(p.out, ob + kHeadDim, lse, p.out_dtype);
+    }
+}
+
 __device__ __forceinline__ float load_any(const void* base, int64_t idx, int dtype) {
     if (dtype == FDK_BF16) return (float)reinterpret_cast<const __bf16*>(base)[idx];
     if (dtype == FDK_FP16) return (float)reinterpret_cast<const _Float16*>(base)[idx];
@@ -128,8 +181,12 @@ __global__ __launch_bounds__(256) void combine_ranks_kernel(const CombineRanksPa
 int launch_combine(const CombineParams& p, hipStream_t stream) {
     const int64_t rows = (int64_t)p.batch * p.hq;
     if (rows == 0) return 0;
-    const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
-    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, p);
+    if (p.num_splits > 8) {
+        hipLaunchKernelGGL(combine_wide_kernel, dim3((unsigned)rows), dim3(256), 0, stream, p);
+    } else {
+        const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
+        hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, stream, p);
+    }
     return (int)hipGetLastError();
 }
 

@@ -84,6 +84,8 @@ int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
 bool mfma_supported(int q_dtype, int kv_dtype, int group);
 int valu_heads_per_wg(int group);
 int mfma_heads_per_wg(int group);
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus);
+int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg);
 
 #if defined(__HIPCC__)
 

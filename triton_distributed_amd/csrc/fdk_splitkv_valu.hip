@@ -1,28 +1,14 @@
 // VALU split kernel: geometry selection and dtype dispatch (kernels: fdk_splitkv_valu.h).
-#include <stdlib.h>
-
 #include "fdk_splitkv_valu.h"
 
 namespace fdk {
 
 namespace {
 
-int env_int(const char* name, int dflt) {
-    const char* s = getenv(name);
-    return (s && *s) ? atoi(s) : dflt;
-}
-
 int pow2_floor(int x) {
     int r = 1;
     while (r * 2 <= x) r *= 2;
     return r;
-}
-
-// kv heads per wave load: a full 1 KB load of adjacent heads when the layout allows it, else one head
-int choose_hs(int hkv, bool heads_contiguous, int kv_dtype) {
-    const int ng = kv_dtype == FDK_FP8_E4M3 ? 8 : 4;
-    if (env_int("FDK_HS", 0) == 1) return 1;
-    return (heads_contiguous && hkv % ng == 0) ? ng : 1;
 }
 
 }  // namespace
@@ -46,9 +32,13 @@ ValuGeometry choose_geometry(const SplitParams& p, int kv_dtype) {
     g.gt = valu_heads_per_wg(p.group);
     g.head_tiles = (p.group + g.gt - 1) / g.gt;
     const bool contiguous = p.k_sh == kHeadDim && p.v_sh == kHeadDim;
-    g.hs = choose_hs(p.hkv, contiguous, kv_dtype);
+    // One kv head per wave load (HS = 1).  The kernel template also supports loads that span several adjacent
+    // heads; on MI355X that variant measured slower for this issue-bound path (fewer, fatter workgroups).
+    g.hs = 1;
+    (void)contiguous;
+    (void)kv_dtype;
     const int n_hg = p.hkv / g.hs;
-    g.nwaves = env_int("FDK_NW", 4) == 8 ? 8 : 4;
+    g.nwaves = 4;
     int per = pow2_floor(n_hg < g.nwaves ? n_hg : g.nwaves);
     while (n_hg % per) per >>= 1;
     g.hg_per_wg = per;

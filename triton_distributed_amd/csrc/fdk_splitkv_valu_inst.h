@@ -31,9 +31,7 @@ int launch_pm(const SplitParams& p, const ValuGeometry& geo, int pm, hipStream_t
 
 template <int QDT, bool FP8, int GT>
 int launch_hs(const SplitParams& p, const ValuGeometry& geo, int pm, hipStream_t stream) {
-    constexpr int NG = Geo<FP8>::NG;
-    if (geo.hs == NG) return launch_pm<QDT, FP8, GT, NG>(p, geo, pm, stream);
-    return launch_pm<QDT, FP8, GT, 1>(p, geo, pm, stream);
+    return launch_pm<QDT, FP8, GT, 1>(p, geo, pm, stream);   // only HS = 1 is instantiated
 }
 
 template <int QDT, bool FP8>
