@@ -37,9 +37,10 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
 #include <stddef.h>
 #include "fdk.h"
 int main(void) {
-  printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
-         offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes));
+         offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
+         offsetof(fdk_decode_args, counters_len));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu\n", sizeof(fdk_plan_t));
@@ -51,7 +52,8 @@ int main(void) {
     lines = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split("\n")
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
-                                       ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes")]
+                                       ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
+                                        "counters_len")]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -134,6 +136,17 @@ def test_workspace_is_required_only_when_the_plan_splits():
     assert _decode_rc(_args(batch=4)) == 0
     # a forced split count needs it as well
     assert _decode_rc(_args(num_splits=4, workspace=None)) == _lib.FDK_EWORKSPACE
+
+
+def test_counters_of_the_work_queue_form():
+    lib = _lib.load()
+    a = _args(batch=4)
+    n = lib.fdk_counters_len(C.byref(a))
+    assert n == 2
+    assert lib.fdk_counters_len(None) == 0
+    # dry run ignores them; a real call would reject a short or misaligned array before launching anything
+    a.counters, a.counters_len = 0x90000, n
+    assert _decode_rc(a) == 0
 
 
 def test_packed_output_needs_a_wider_row():

@@ -275,6 +275,29 @@ def test_split_then_combine_entry_points_equal_the_fused_call(cuda_device):
         torch.testing.assert_close(l, ref_l, atol=1e-5, rtol=0)
 
 
+@pytest.mark.parametrize("config,kw", [("ragged_g8", dict(batch=40, kv_len_range=(1, 6000))),
+                                       ("llama3_8b_b32", dict(batch=3, kv_len=3000))])
+def test_work_queue_form_equals_one_workgroup_per_item_and_restores_its_counters(cuda_device, config, kw):
+    # a fixed set of workgroups pulling items from a queue against one workgroup per item
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS[config], **kw), cuda_device, poison_tail=True)
+    for kv_split in (-1, 7, 64):
+        two = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                 kv_split=kv_split, work_queue=False)
+        ctr = torch.zeros(8, dtype=torch.int32, device=cuda_device)
+        one = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                 kv_split=kv_split, counters=ctr)
+        assert one.plan.num_splits == two.plan.num_splits
+        o2, l2 = two.run()
+        for _ in range(3):                               # repeated calls reuse the same counters
+            one.out.zero_()
+            o1, l1 = one.run()
+        torch.cuda.synchronize()
+        assert torch.equal(o1, o2) and torch.equal(l1, l2)     # same items, same arithmetic, same merge
+        assert int(ctr.abs().sum()) == 0
+        _check(o1, l1, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
+               tag=f"work queue S={kv_split}")
+
+
 def test_runs_on_a_side_stream_and_is_repeatable(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=4, kv_len=1500), cuda_device)
     call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)

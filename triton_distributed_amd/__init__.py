@@ -1,25 +1,28 @@
 """MI355X-native flash-decode: split-KV paged GQA decode attention + LSE combine (gfx950 HIP kernels).
 
-Importing this package loads ``lib/libfdk.so``; it raises ImportError if the library has not been built
-(``python -m triton_distributed_amd.build``).  There is no CPU or eager fallback.
+The entry points live in ``flash_decode`` and are loaded on first use; that loads ``lib/libfdk.so`` and raises
+ImportError if the library has not been built (``python -m triton_distributed_amd.build``) or does not match
+this package's ABI version.  There is no CPU or eager fallback.  ``triton_distributed_amd.build`` itself
+imports without the library.
 """
-from .flash_decode import (  # noqa: F401
-    PreparedDecode,
-    SplitKvPlan,
-    flash_decode,
-    get_split_kv_plan,
-    gqa_fwd_batch_decode,
-    gqa_fwd_batch_decode_aot,
-    gqa_fwd_batch_decode_intra_rank,
-    gqa_fwd_batch_decode_intra_rank_aot,
-    inter_rank_combine,
-    pack_out_lse,
-    prepare_decode,
-    unpack_out_lse,
-)
+import importlib
 
 __all__ = [
     "PreparedDecode", "SplitKvPlan", "flash_decode", "get_split_kv_plan", "gqa_fwd_batch_decode",
     "gqa_fwd_batch_decode_aot", "gqa_fwd_batch_decode_intra_rank", "gqa_fwd_batch_decode_intra_rank_aot",
     "inter_rank_combine", "pack_out_lse", "prepare_decode", "unpack_out_lse",
 ]
+
+
+def __getattr__(name):
+    if name in __all__:
+        mod = importlib.import_module(".flash_decode", __name__)     # loads libfdk.so; raises if it is missing
+        # bind every entry point on the package (the function ``flash_decode`` takes the place of the
+        # submodule attribute of the same name that the import just set)
+        globals().update({n: getattr(mod, n) for n in __all__})
+        return globals()[name]
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+
+
+def __dir__():
+    return sorted(list(globals()) + __all__)

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 1
+FDK_ABI_VERSION = 2
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -24,7 +24,7 @@ FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN = 1, 2
 
 EXPORTS = (
     "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
-    "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks",
+    "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len",
 )
 
 
@@ -49,6 +49,7 @@ class FdkDecodeArgs(C.Structure):
         ("out_dtype", C.c_int32), ("algo", C.c_int32),
         ("lse", C.c_void_p), ("lse_stride_b", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("counters", C.c_void_p), ("counters_len", C.c_int64),
     ]
 
 
@@ -103,6 +104,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(FdkDecodeArgs), C.c_void_p]
+    lib.fdk_counters_len.restype = C.c_int64
+    lib.fdk_counters_len.argtypes = [C.POINTER(FdkDecodeArgs)]
     lib.fdk_combine_ranks.restype = C.c_int
     lib.fdk_combine_ranks.argtypes = [C.POINTER(FdkCombineRanksArgs), C.c_void_p]
     if lib.fdk_abi_version() != FDK_ABI_VERSION:

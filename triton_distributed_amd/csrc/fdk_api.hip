@@ -221,6 +221,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.v_scale = a->kv_dtype == FDK_FP8_E4M3 ? a->v_scale : nullptr;
     sp.part_o = part_o; sp.part_lse = part_lse;
     sp.out = a->out; sp.lse = a->lse;
+    sp.counters = nullptr;
+    sp.num_cus = query_cus();
     sp.q_sb = a->q_stride_b; sp.q_sh = a->q_stride_h;
     sp.k_sp = a->k_stride_page; sp.k_st = a->k_stride_tok; sp.k_sh = a->k_stride_head;
     sp.v_sp = a->v_stride_page; sp.v_st = a->v_stride_tok; sp.v_sh = a->v_stride_head;
@@ -269,6 +271,11 @@ const char* fdk_last_error(void) { return g_err; }
 
 int fdk_device_cus(void) { return query_cus(); }
 
+int64_t fdk_counters_len(const fdk_decode_args* a) {
+    if (!a || a->batch <= 0 || a->num_q_heads <= 0) return 0;
+    return 2;      // queue head, finished-workgroup count
+}
+
 size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim, int32_t num_splits) {
     if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 0) return 0;
     const size_t rows = (size_t)batch * (size_t)num_q_heads * (size_t)num_splits;
@@ -306,6 +313,15 @@ int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
     rc = resolve(args, true, &r);
     if (rc) return rc;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
+    // work-queue form of the split kernel (matrix-core path only)
+    const bool queued = !r.sp.direct && args->counters != nullptr && r.plan.algo == FDK_ALGO_MFMA;
+    if (queued) {
+        if (reinterpret_cast<uintptr_t>(args->counters) & 3u) return fail(FDK_EALIGN, "counters not 4-byte aligned");
+        if (args->counters_len < fdk_counters_len(args))
+            return fail(FDK_EWORKSPACE, "counters_len %lld < %lld", (long long)args->counters_len,
+                        (long long)fdk_counters_len(args));
+        r.sp.counters = args->counters;
+    }
     rc = launch_split(args, r, stream);
     if (rc) return rc;
     if (!r.sp.direct) {

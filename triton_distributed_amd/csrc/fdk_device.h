@@ -27,6 +27,7 @@ struct SplitParams {
     float* part_lse;  // [B, Hq, S]    fp32 (S > 1)
     void* out;        // final output, written directly when S == 1
     float* lse;       // may be null
+    int32_t* counters;  // zeroed scratch counters of the work queue: [0] head, [1] finished workgroups
     int64_t q_sb, q_sh;
     int64_t k_sp, k_st, k_sh;  // page / token / head strides, elements
     int64_t v_sp, v_st, v_sh;
@@ -41,6 +42,7 @@ struct SplitParams {
     int32_t out_dtype;              // fdk_dtype
     int32_t pack_lse;
     int32_t direct;                 // 1: single split, write the final (out, lse) instead of partials
+    int32_t persistent, total_items, num_cus;
     float scale_log2;               // sm_scale * log2(e)
     float soft_cap;                 // > 0: on (applied to natural-unit logits)
     float sm_scale;

@@ -109,7 +109,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     float* sm_m = reinterpret_cast<float*>(lds + nw * kScratch);
     float* sm_l = sm_m + nw * 16;
 
-    int wg = blockIdx.x;
+    int* const s_next = reinterpret_cast<int*>(sm_l + nw * 16);     // next work item (persistent mode)
+
+    // ---- one work item: (sequence, split, kv-head block, q-head tile) ------------------------------------------
+    auto run_item = [&](int wg) {
     const int ht = wg % p.head_tiles;
     wg /= p.head_tiles;
     const int hgb = wg % p.hg_blocks;
@@ -120,8 +123,23 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     const int head0 = kvh * p.group + ht * 16;
     const int heads_here = min(16, p.group - ht * 16);
 
-    const int kv_len = min(p.kv_lens[b], p.max_tokens);
+    // Issue everything that does not depend on kv_len first, so that the dependent chain before the first K/V
+    // load is as short as possible: Q^T (the B operand of S^T = K Q^T: lane (h = c, a) holds
+    // q[h][32 ks + 8 a .. +7]; columns past the group repeat its last head - their results are never stored,
+    // and nothing waits for a select) and, speculatively, the page of this wave's first tile (any table column
+    // may be read; the value is used only if the tile exists).
+    uint4 qb[4];
+    {
+        const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
+                             (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+    }
+    const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
     const int c_start = split * p.chunk;
+    int first_pg = 0;
+    if (PM == PM_TILE) first_pg = tbl[min(c_start + tix * kTile, p.max_tokens - 1) >> p.page_shift];
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
     if (c_start >= kv_len) {
         if (p.direct && tix == 0) {   // kv_len == 0 with a single split: defined result, no combine follows
             for (int idx = lane; idx < heads_here * kHeadDim; idx += 64) {
@@ -148,7 +166,6 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     const char* kbase = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES + lpiece * 16;
     const char* vbase = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES + lpiece * 16;
-    const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
     const int pmask = p.page_size - 1;
     char* my_lds = lds + wave * kScratch;
     char* lds_k = my_lds;
@@ -208,7 +225,6 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         }
     };
 
-    uint4 qb[4];                                 // Q^T operand, loaded after the first tile's loads are on their way
     float m_run = -INFINITY, l_run = 0.f;       // for head c; l_run is this lane group's share of the sum
     f32x4_t acc[8];                              // acc[db][i] = O[h = c][16 db + 4 a + i]
 #pragma unroll
@@ -314,17 +330,9 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         int t = tix;
         const int st = ti_n;
         if (t < n_full) {
-            pages_of(t, pid);
+            if (PM == PM_TILE) pid.pg[0] = first_pg; else pages_of(t, pid);
             issue_full(t, pid, rg);
             if (t + st < n_full) pages_of(t + st, pid);
-        }
-        // Q^T as the B operand of S^T = K Q^T: lane (h = c, a) holds q[h][32 ks + 8 a .. +7].  Columns past
-        // the group repeat its last head: their results are never stored, and nothing waits for a select.
-        {
-            const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
-                                 (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
         }
         if (NBUF == 1) {
             // one register buffer: the next tile's loads go into the registers just staged
@@ -414,6 +422,28 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             if (d == 0) p.part_lse[row] = lse_nat;
         }
     }
+
+    };   // run_item
+
+    // ---- work distribution: one item per workgroup, or (persistent) a fixed set of workgroups that pull items
+    // from a queue: counters[0] is its head, counters[1] counts finished workgroups; the last one to finish
+    // puts both back to zero.  The first item of every workgroup is its own index.
+    int item = blockIdx.x;
+    while (item < p.total_items) {
+        run_item(item);
+        if (!p.persistent) return;
+        __syncthreads();
+        if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
+        __syncthreads();
+        item = s_next[0];
+    }
+    if (threadIdx.x == 0) {
+        const int done = atomicAdd(p.counters + 1, 1);
+        if (done == (int)gridDim.x - 1) {
+            atomicExch(p.counters, 0);
+            atomicExch(p.counters + 1, 0);
+        }
+    }
 }
 
 template <int QDT, bool FP8>
@@ -423,14 +453,19 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     if (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) p.hg_per_wg = 1;
     p.hg_blocks = p.hkv / p.hg_per_wg;
     const int nw = p.hg_per_wg > 4 ? p.hg_per_wg : 4;
-    const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float));
+    const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float)) + 16;
     constexpr int RPL = FP8 ? 8 : 4;
     int pm;
     if (p.page_shift < 0) pm = PM_LANE_DIV;
     else if (p.page_size % kTile == 0) pm = PM_TILE;
     else if (p.page_size % RPL == 0) pm = PM_LOAD;
     else pm = PM_LANE;
-    const dim3 grid((unsigned)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles));
+    p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
+    // Persistent mode (work queue) whenever the KV range is split and the caller provided counters: items of a
+    // ragged batch differ in length, and a queue keeps every compute unit busy until the end.
+    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
+    p.persistent = (p.counters != nullptr && !p.direct && p.total_items > resident) ? 1 : 0;
+    const dim3 grid((unsigned)(p.persistent ? resident : p.total_items));
     const dim3 block(64 * nw);
     const int nbuf = 2;
 #define FDK_MFMA_LAUNCH(PMV)                                                                                         \

@@ -157,6 +157,22 @@ def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, s
     return _plan_of(a, num_cus)
 
 
+_COUNTER_CACHE = {}
+
+
+def _stream_counters(device: torch.device, stream, n: int = 64) -> torch.Tensor:
+    """Zeroed int32 counters shared by the calls issued on one stream (they run in order, and every call
+    leaves the counters zero), so the convenience entry points need no fill launch per call."""
+    if device.type != "cuda":
+        return None                                   # the caller is about to be told that there is no CPU path
+    key = (device.index, _stream_handle(stream))
+    t = _COUNTER_CACHE.get(key)
+    if t is None or t.numel() < n:
+        t = torch.zeros(n, dtype=torch.int32, device=device)
+        _COUNTER_CACHE[key] = t
+    return t
+
+
 class PreparedDecode:
     """A fully bound decode call: arguments marshalled once, ``run()`` only enqueues the kernels.
 
@@ -185,11 +201,15 @@ class PreparedDecode:
 
 def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
-                   algo="auto", packed_out=None, want_lse=True, always_workspace=False) -> PreparedDecode:
+                   algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
+                   work_queue=True) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
-    dtype) in ``[..., D]`` - the reference's ``output_combine`` layout - instead of ``out``."""
+    dtype) in ``[..., D]`` - the reference's ``output_combine`` layout - instead of ``out``.
+    ``counters``: zeroed int32 tensor for the work-queue form of a split decode (a fixed set of workgroups pulls
+    the work items, which keeps ragged batches balanced); by default the call owns a private one.
+    ``work_queue=False`` launches one workgroup per item instead."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -229,7 +249,18 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         a.workspace = workspace.data_ptr()
         a.workspace_bytes = workspace.numel() * workspace.element_size()
-    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace)
+    if plan.num_splits > 1 and plan.algo == "mfma" and work_queue:
+        n_ctr = int(_LIB.fdk_counters_len(C.byref(a)))
+        if counters is None:
+            counters = torch.zeros(n_ctr, dtype=torch.int32, device=q.device)
+        elif counters.dtype != torch.int32 or counters.numel() < n_ctr or not counters.is_cuda or \
+                not counters.is_contiguous():
+            raise ValueError(f"counters must be a contiguous int32 GPU tensor of at least {n_ctr} zeros")
+        a.counters = counters.data_ptr()
+        a.counters_len = counters.numel()
+    else:
+        counters = None
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, counters)
     return PreparedDecode(a, plan, keep, target, lse)
 
 
@@ -257,7 +288,8 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     and lse = ln sum exp(scaled logits) - what the cross-rank combine consumes."""
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
-                          out=out, lse=lse, workspace=workspace, algo=algo)
+                          out=out, lse=lse, workspace=workspace, algo=algo,
+                          counters=_stream_counters(q.device, stream))
     return call.run(stream)
 
 
@@ -273,7 +305,7 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
         output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
-                          want_lse=False)
+                          want_lse=False, counters=_stream_counters(q.device, stream))
     call.run(stream)
     return output_combine
 
@@ -283,7 +315,7 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
     """Drop-in for the reference function of the same name (flash_decode.py:763-844): ``[B, Hq, D]``."""
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
-                          want_lse=False)
+                          want_lse=False, counters=_stream_counters(q.device, stream))
     return call.run(stream)[0]
 
 
