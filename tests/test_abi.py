@@ -111,8 +111,8 @@ def test_valid_arguments_pass_dry_run():
     ("table_stride_b", 255, _lib.FDK_ESHAPE),
     ("out_stride_h", 127, _lib.FDK_ESHAPE),
     ("num_splits", 5000, _lib.FDK_ESHAPE),
-    ("head_dim", 256, _lib.FDK_EUNSUPPORTED),
-    ("head_dim", 64, _lib.FDK_EUNSUPPORTED),
+    ("head_dim", 96, _lib.FDK_EUNSUPPORTED),
+    ("head_dim", 512, _lib.FDK_EUNSUPPORTED),
     ("q_dtype", _lib.FDK_FP32, _lib.FDK_EUNSUPPORTED),
     ("kv_dtype", _lib.FDK_FP16, _lib.FDK_EUNSUPPORTED),
     ("out_dtype", _lib.FDK_FP8_E4M3, _lib.FDK_EUNSUPPORTED),
@@ -179,13 +179,15 @@ def test_plan_scales_splits_with_occupancy():
     p4 = _plan(_args(batch=4))
     assert p4.num_splits > 1 and p4.chunk_tokens % 64 == 0
     assert p4.num_splits * p4.chunk_tokens >= 4096 > (p4.num_splits - 1) * p4.chunk_tokens
-    # few units, long context -> many splits; chunks never shorter than 256 tokens
+    # few units, long context -> many splits; chunks of a long context are never shorter than 512 tokens
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
                          q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
-    assert p_long.num_splits > p4.num_splits and p_long.chunk_tokens >= 512
-    # short context is never split below the minimum chunk
+    assert p_long.num_splits >= p4.num_splits and p_long.chunk_tokens >= 512 > p4.chunk_tokens
+    # a short context is latency-bound: it is split down to chunks of 64 tokens, never finer
     p_short = _plan(_args(batch=1, max_pages=8, table_stride_b=8))
-    assert p_short.num_splits == 1 and p_short.chunk_tokens >= 128
+    assert p_short.num_splits == 2 and p_short.chunk_tokens == 64
+    p_one = _plan(_args(batch=1, max_pages=4, table_stride_b=4))
+    assert p_one.num_splits == 1 and p_one.chunk_tokens == 64
     # the host's bound on kv_len drives the split, not the table width
     p_hint = _plan(_args(batch=4, max_pages=2048, table_stride_b=2048, max_kv_len=4096))
     assert (p_hint.num_splits, p_hint.chunk_tokens) == (p4.num_splits, p4.chunk_tokens)

@@ -104,12 +104,74 @@ def test_large_pool_index_arithmetic(cuda_device):
     _check(out, lse, q, k, v, table, lens, d ** -0.5, tag="bigpool")
 
 
-def test_head_dim_256_is_rejected(cuda_device):
-    q = torch.zeros(1, 8, 256, dtype=torch.float16, device=cuda_device)
-    k = torch.zeros(4, 16, 8, 256, dtype=torch.float16, device=cuda_device)
-    with pytest.raises(ValueError, match="head_dim"):
-        tda.flash_decode(q, k, k, torch.zeros(1, 1, dtype=torch.int32, device=cuda_device),
-                         _lens_t([1], cuda_device), 1.0)
+def test_unbuilt_head_dims_are_rejected(cuda_device):
+    tbl = torch.zeros(1, 1, dtype=torch.int32, device=cuda_device)
+    for d, algo in ((96, "auto"), (512, "auto"), (256, "valu"), (64, "valu")):
+        q = torch.zeros(1, 8, d, dtype=torch.float16, device=cuda_device)
+        k = torch.zeros(4, 16, 8, d, dtype=torch.float16, device=cuda_device)
+        with pytest.raises(ValueError, match="head_dim"):
+            tda.flash_decode(q, k, k, tbl, _lens_t([1], cuda_device), 1.0, algo=algo)
+
+
+# ---- head sizes other than 128: 256 is in the reference's grid (test_decode_attn.py:125), 64 is built as well ----
+@pytest.mark.parametrize("head_size", [64, 256])
+@pytest.mark.parametrize("kv_lens", [[1320, 18, 463], [1, 54, 293, 70]])
+@pytest.mark.parametrize("num_heads", [(16, 16), (32, 8), (64, 8), (6, 1)])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("soft_cap", [0, 50])
+def test_reference_grid_other_head_sizes(cuda_device, head_size, kv_lens, num_heads, block_size, dtype, soft_cap):
+    print(f"case D={head_size} lens={kv_lens} heads={num_heads} P={block_size} {dtype} cap={soft_cap}", flush=True)
+    num_blocks = 512
+    g = torch.Generator(device="cpu").manual_seed(hash((head_size, tuple(kv_lens), num_heads, block_size)) & 0xFFFF)
+    hq, hkv = num_heads
+    d = head_size
+    scale = d ** -0.5
+    q = torch.randn(len(kv_lens), hq, d, generator=g).to(dtype).to(cuda_device)
+    kv = torch.randn(num_blocks + 1, 2, block_size, hkv, d, generator=g).to(dtype).to(cuda_device)
+    k, v = kv[:, 0], kv[:, 1]
+    max_blocks = (max(kv_lens) + block_size - 1) // block_size
+    table = torch.randint(0, num_blocks, (len(kv_lens), max_blocks), generator=g, dtype=torch.int32).to(cuda_device)
+    lens_t = _lens_t(kv_lens, cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap))
+    out1, lse1 = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap), kv_split=1)
+    out9, lse9 = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap), kv_split=9)
+    packed = tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale,
+                                                 float(soft_cap), kv_split=32)
+    torch.cuda.synchronize()
+    for o, l, tag in ((out, lse, "auto"), (out1, lse1, "S=1"), (out9, lse9, "S=9")):
+        _check(o, l, q, k, v, table, kv_lens, scale, float(soft_cap), tag=f"D={d} {tag}")
+    assert packed.shape == (len(kv_lens), hq, d + 1) and packed.dtype == dtype
+    torch.testing.assert_close(packed[..., :d].float(), out.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(packed[..., d].float(), lse, atol=3e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("head_size", [64, 256])
+@pytest.mark.parametrize("page", [16, 4, 6, 64])
+def test_other_head_sizes_fp8_pages_and_rank_merge(cuda_device, head_size, page):
+    d = head_size
+    cfg = wl.DecodeConfig("fp8_d", 57 + d + page, 5, 32, 8, d, page, kv_len_range=(1, 1500), kv_dtype="fp8_e4m3",
+                          spare_pages=4)
+    inp = wl.make_inputs(cfg, cuda_device, poison_tail=True)
+    out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                k_scale=inp.k_scale, v_scale=inp.v_scale)
+    torch.cuda.synchronize()
+    kd = ofp8.dequant_per_head(inp.k_cache, inp.k_scale)
+    vd = ofp8.dequant_per_head(inp.v_cache, inp.v_scale)
+    _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
+           ref_kv=(kd, vd), tag=f"fp8 D={d} P={page}")
+    # bf16 cache of the same shape, then the cross-rank merge of two copies of the result: merging a result
+    # with itself leaves out unchanged and adds ln 2 to lse
+    o2, l2 = tda.flash_decode(inp.q, kd, vd, inp.block_table, inp.kv_lens, inp.sm_scale)
+    torch.cuda.synchronize()
+    _check(o2, l2, inp.q, kd, vd, inp.block_table, inp.kv_lens_host, inp.sm_scale, tag=f"bf16 D={d} P={page}")
+    both = torch.stack([tda.pack_out_lse(o2, l2, torch.float32)] * 2)
+    gl = inp.kv_lens[None].repeat(2, 1)
+    lse_m = torch.empty_like(l2)
+    merged = tda.inter_rank_combine(both, gl, lse_out=lse_m)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(merged.float(), o2.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse_m, l2 + math.log(2.0), atol=1e-4, rtol=0)
 
 
 # ---- golden vectors and edge cases -----------------------------------------------------------------------------

@@ -38,9 +38,13 @@ def test_shape_and_dtype_checks_mirror_the_reference_asserts():
         tda.get_split_kv_plan(q, k, v, table[:1], lens)
     with pytest.raises(ValueError):
         tda.get_split_kv_plan(q.float(), k, v, table, lens)
-    with pytest.raises(ValueError):                           # head_dim 256 is in the reference grid, not built here
-        q2, k2, v2, t2, l2 = _cpu_inputs(d=256)
-        tda.get_split_kv_plan(q2, k2, v2, t2, l2)
+    q2, k2, v2, t2, l2 = _cpu_inputs(d=256)                   # head_dim 256 is in the reference grid
+    assert tda.get_split_kv_plan(q2, k2, v2, t2, l2).algo == "mfma"
+    with pytest.raises(ValueError):                           # the vector path is built for head_dim 128 only
+        tda.get_split_kv_plan(q2, k2, v2, t2, l2, algo="valu")
+    with pytest.raises(ValueError):
+        q3, k3, v3, t3, l3 = _cpu_inputs(d=96)
+        tda.get_split_kv_plan(q3, k3, v3, t3, l3)
     with pytest.raises(ValueError):
         tda.get_split_kv_plan(q.transpose(1, 2).contiguous().transpose(1, 2), k, v, table, lens)
 

@@ -58,7 +58,8 @@ int query_cus() {
 }
 
 constexpr int kChunkAlign = 64;     // split boundaries fall on multiples of 64 tokens
-constexpr int kMinChunk = 512;      // never split finer than this
+constexpr int kMinChunk = 64;       // shortest chunk (short contexts: latency matters more than the partials)
+constexpr int kMaxMinChunk = 512;   // long contexts are never split finer than this
 constexpr int kMaxSplits = 1024;
 
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
@@ -70,8 +71,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         return fail(FDK_ESHAPE, "head counts must be positive (Hq=%d, Hkv=%d)", a->num_q_heads, a->num_kv_heads);
     if (a->num_q_heads % a->num_kv_heads != 0)
         return fail(FDK_ESHAPE, "Hq=%d not a multiple of Hkv=%d", a->num_q_heads, a->num_kv_heads);
-    if (a->head_dim != fdk::kHeadDim)
-        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (only %d)", a->head_dim, fdk::kHeadDim);
+    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
+        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
     if (a->page_size <= 0) return fail(FDK_ESHAPE, "page_size %d <= 0", a->page_size);
     if (a->max_pages <= 0) return fail(FDK_ESHAPE, "max_pages %d <= 0", a->max_pages);
     if ((int64_t)a->max_pages * a->page_size > INT32_MAX)
@@ -102,8 +103,9 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         if (ks[i] < 0) return fail(FDK_ESHAPE, "negative cache stride");
         if ((ks[i] * kes) % 16) return fail(FDK_EALIGN, "cache strides must be multiples of 16 bytes");
     }
-    if (a->k_stride_head < fdk::kHeadDim && a->num_kv_heads > 1)
-        return fail(FDK_ESHAPE, "k head stride %lld < head_dim", (long long)a->k_stride_head);
+    if ((a->k_stride_head < a->head_dim || a->v_stride_head < a->head_dim) && a->num_kv_heads > 1)
+        return fail(FDK_ESHAPE, "cache head stride < head_dim (k %lld, v %lld)", (long long)a->k_stride_head,
+                    (long long)a->v_stride_head);
     if (a->table_stride_b < a->max_pages)
         return fail(FDK_ESHAPE, "table_stride_b %lld < max_pages %d", (long long)a->table_stride_b, a->max_pages);
 
@@ -113,7 +115,7 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         if (a->out_dtype != FDK_BF16 && a->out_dtype != FDK_FP16 && a->out_dtype != FDK_FP32)
             return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);
         if (reinterpret_cast<uintptr_t>(a->out) % oes) return fail(FDK_EALIGN, "out not element aligned");
-        const int row = fdk::kHeadDim + ((a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0);
+        const int row = a->head_dim + ((a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0);
         if (a->out_stride_h < row) return fail(FDK_ESHAPE, "out_stride_h %lld < %d", (long long)a->out_stride_h, row);
         if (a->lse && (reinterpret_cast<uintptr_t>(a->lse) & 3u)) return fail(FDK_EALIGN, "lse not 4-byte aligned");
         if (a->lse && a->lse_stride_b < a->num_q_heads)
@@ -129,13 +131,14 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     if (algo == FDK_ALGO_AUTO) {
         // The matrix-core path is the default for every group size: on MI355X it is at least as fast as the
         // vector path even for small groups, because it needs an order of magnitude fewer issue slots per KV byte.
-        algo = fdk::mfma_supported(a->q_dtype, a->kv_dtype, group) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
+        algo = fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
     }
-    if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group))
-        return fail(FDK_EUNSUPPORTED, "MFMA path not built for q_dtype=%d kv_dtype=%d group=%d", a->q_dtype,
-                    a->kv_dtype, group);
-    if (algo == FDK_ALGO_VALU && !fdk::valu_supported(a->q_dtype, a->kv_dtype, group))
-        return fail(FDK_EUNSUPPORTED, "VALU path not built for q_dtype=%d kv_dtype=%d", a->q_dtype, a->kv_dtype);
+    if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim))
+        return fail(FDK_EUNSUPPORTED, "MFMA path not built for q_dtype=%d kv_dtype=%d head_dim=%d", a->q_dtype,
+                    a->kv_dtype, a->head_dim);
+    if (algo == FDK_ALGO_VALU && !fdk::valu_supported(a->q_dtype, a->kv_dtype, group, a->head_dim))
+        return fail(FDK_EUNSUPPORTED, "VALU path not built for q_dtype=%d kv_dtype=%d head_dim=%d (128 only)", a->q_dtype,
+                    a->kv_dtype, a->head_dim);
 
     int64_t max_len = a->max_kv_len > 0 ? a->max_kv_len : (int64_t)a->max_pages * a->page_size;
     const int64_t table_cap = (int64_t)a->max_pages * a->page_size;
@@ -144,7 +147,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
 
     if (num_cus <= 0) num_cus = query_cus();
     const int batch = a->batch > 0 ? a->batch : 1;
-    const bool heads_contiguous = a->k_stride_head == fdk::kHeadDim && a->v_stride_head == fdk::kHeadDim;
+    const bool heads_contiguous = a->k_stride_head == a->head_dim && a->v_stride_head == a->head_dim;
     int kv_heads_per_wg = 1;
     int units_per_seq;
     if (algo == FDK_ALGO_MFMA) {
@@ -156,8 +159,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const int64_t units = (int64_t)batch * units_per_seq;
 
     // Split count: none when the (sequence, head block) units alone fill the compute units - a single pass
-    // then writes the final result and no combine runs.  Otherwise aim at two workgroups per compute unit,
-    // with chunks of at least kMinChunk tokens.
+    // then writes the final result and no combine runs.  Otherwise aim at two workgroups per compute unit.
+    // The shortest chunk grows with the context (max_len / 64, between kMinChunk and kMaxMinChunk tokens):
+    // a short context is latency-bound and gains from every extra split, a long one pays for each partial
+    // row it writes and re-reads.
     int64_t splits;
     if (a->num_splits > 0) {
         splits = a->num_splits;
@@ -165,7 +170,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         splits = 1;
     } else {
         splits = cdiv64(2 * (int64_t)num_cus, units);
-        const int64_t cap = cdiv64(max_len, kMinChunk);
+        int64_t min_chunk = cdiv64(cdiv64(max_len, 64), kChunkAlign) * kChunkAlign;
+        if (min_chunk < kMinChunk) min_chunk = kMinChunk;
+        if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
+        const int64_t cap = cdiv64(max_len, min_chunk);
         if (splits > cap) splits = cap;
         if (splits < 1) splits = 1;
     }
@@ -211,7 +219,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
         if (a->workspace_bytes < need)
             return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed for %d splits", a->workspace_bytes, need, S);
         part_o = reinterpret_cast<float*>(a->workspace);
-        part_lse = part_o + rows * S * fdk::kHeadDim;
+        part_lse = part_o + rows * S * a->head_dim;
     }
     fdk::SplitParams& sp = r->sp;
     memset(&sp, 0, sizeof(sp));
@@ -230,6 +238,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.out_sb = a->out_stride_b; sp.out_sh = a->out_stride_h; sp.lse_sb = a->lse_stride_b;
     sp.batch = a->batch; sp.hq = a->num_q_heads; sp.hkv = a->num_kv_heads;
     sp.group = a->num_q_heads / a->num_kv_heads;
+    sp.head_dim = a->head_dim;
     sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
     sp.num_splits = S; sp.chunk = r->plan.chunk_tokens;
     sp.max_tokens = (int32_t)((int64_t)a->max_pages * a->page_size);
@@ -247,7 +256,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     cp.part_o = part_o; cp.part_lse = part_lse; cp.kv_lens = a->kv_lens;
     cp.out = a->out; cp.lse = a->lse;
     cp.out_sb = a->out_stride_b; cp.out_sh = a->out_stride_h; cp.lse_sb = a->lse_stride_b;
-    cp.batch = a->batch; cp.hq = a->num_q_heads;
+    cp.batch = a->batch; cp.hq = a->num_q_heads; cp.head_dim = a->head_dim;
     cp.num_splits = S; cp.chunk = r->plan.chunk_tokens;
     cp.max_tokens = sp.max_tokens;
     cp.out_dtype = a->out_dtype; cp.pack_lse = sp.pack_lse;
@@ -362,15 +371,16 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
         return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_combine_ranks_args));
     if (a->num_ranks <= 0 || a->batch < 0 || a->num_q_heads <= 0)
         return fail(FDK_ESHAPE, "bad dims R=%d B=%d Hq=%d", a->num_ranks, a->batch, a->num_q_heads);
-    if (a->head_dim != fdk::kHeadDim) return fail(FDK_EUNSUPPORTED, "head_dim %d not built", a->head_dim);
+    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
+        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
     const bool packed = (a->flags & FDK_FLAG_PACK_LSE) != 0;
     if (elem_size(a->partial_dtype) < 2) return fail(FDK_EUNSUPPORTED, "partial_dtype %d", a->partial_dtype);
     if (elem_size(a->out_dtype) < 2) return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);
     if (a->batch == 0) return FDK_OK;
     if (!a->partial || !a->kv_lens || !a->out) return fail(FDK_ENULL, "partial / kv_lens / out must be non-null");
     if (!packed && !a->partial_lse) return fail(FDK_ENULL, "partial_lse is null and FDK_FLAG_PACK_LSE is not set");
-    if (a->stride_h < fdk::kHeadDim + (packed ? 1 : 0)) return fail(FDK_ESHAPE, "stride_h too small");
-    if (a->out_stride_h < fdk::kHeadDim) return fail(FDK_ESHAPE, "out_stride_h too small");
+    if (a->stride_h < a->head_dim + (packed ? 1 : 0)) return fail(FDK_ESHAPE, "stride_h too small");
+    if (a->out_stride_h < a->head_dim) return fail(FDK_ESHAPE, "out_stride_h too small");
     if (a->flags & FDK_FLAG_DRY_RUN) return FDK_OK;
     fdk::CombineRanksParams p;
     memset(&p, 0, sizeof(p));
@@ -379,7 +389,7 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
     p.stride_r = a->stride_r; p.stride_b = a->stride_b; p.stride_h = a->stride_h;
     p.lse_stride_r = a->lse_stride_r; p.lse_stride_b = a->lse_stride_b;
     p.out_sb = a->out_stride_b; p.out_sh = a->out_stride_h; p.lse_sb_out = a->lse_stride_b_out;
-    p.num_ranks = a->num_ranks; p.batch = a->batch; p.hq = a->num_q_heads;
+    p.num_ranks = a->num_ranks; p.batch = a->batch; p.hq = a->num_q_heads; p.head_dim = a->head_dim;
     p.partial_dtype = a->partial_dtype; p.out_dtype = a->out_dtype; p.packed = packed ? 1 : 0;
     int rc = fdk::launch_combine_ranks(p, reinterpret_cast<hipStream_t>(hip_stream));
     if (rc) return fail(rc, "rank combine launch failed: %s", hipGetErrorString((hipError_t)rc));

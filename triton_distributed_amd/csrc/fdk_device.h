@@ -8,7 +8,7 @@
 
 namespace fdk {
 
-constexpr int kHeadDim = 128;       // the only head dimension built
+constexpr int kHeadDim = 128;       // head dimension of the vector path (the matrix-core path: 64, 128, 256)
 constexpr int kWaveSize = 64;
 constexpr int kWavesPerWg = 4;      // split kernels run 256-thread workgroups
 constexpr float kLog2e = 1.4426950408889634f;
@@ -33,7 +33,7 @@ struct SplitParams {
     int64_t v_sp, v_st, v_sh;
     int64_t tbl_sb;
     int64_t out_sb, out_sh, lse_sb;
-    int32_t batch, hq, hkv, group;
+    int32_t batch, hq, hkv, group, head_dim;
     int32_t page_size, page_shift;  // page_shift = log2(page_size) or -1
     int32_t num_splits, chunk;
     int32_t max_tokens;             // block_table columns * page_size: kv_len is clamped to it
@@ -55,7 +55,7 @@ struct CombineParams {
     void* out;
     float* lse;
     int64_t out_sb, out_sh, lse_sb;
-    int32_t batch, hq;
+    int32_t batch, hq, head_dim;
     int32_t num_splits, chunk;
     int32_t max_tokens;
     int32_t out_dtype;
@@ -71,7 +71,7 @@ struct CombineRanksParams {
     int64_t stride_r, stride_b, stride_h;
     int64_t lse_stride_r, lse_stride_b;
     int64_t out_sb, out_sh, lse_sb_out;
-    int32_t num_ranks, batch, hq;
+    int32_t num_ranks, batch, hq, head_dim;
     int32_t partial_dtype, out_dtype, packed;
 };
 
@@ -80,10 +80,10 @@ int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStre
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_combine(const CombineParams& p, hipStream_t stream);
 int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
-bool valu_supported(int q_dtype, int kv_dtype, int group);
+bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);
 // workgroups per (sequence, split) of the VALU path for this head layout
 int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
-bool mfma_supported(int q_dtype, int kv_dtype, int group);
+bool mfma_supported(int q_dtype, int kv_dtype, int group, int head_dim);
 int valu_heads_per_wg(int group);
 int mfma_heads_per_wg(int group);
 int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus);

@@ -1,0 +1,507 @@
+// Split-KV paged GQA decode, matrix-core path, gfx950: the kernel template (one translation unit per head
+// dimension instantiates it).
+//
+// Same contract as the vector-ALU kernel (fdk_splitkv_valu.h) and the same counterpart in the reference
+// (kernel_gqa_fwd_batch_decode_split_kv, python/triton_dist/kernels/nvidia/flash_decode.py:129-239, which
+// pads the q-head group to a 16-row tile for its tl.dot, :170-176).  One workgroup per (sequence, split,
+// block of kv heads, tile of 16 q heads).  Each wavefront owns one kv head; a workgroup covers up to eight
+// adjacent kv heads, so that together its wavefronts stream whole token rows (all heads of a token are
+// adjacent in the cache) - a compute unit then reads contiguous memory, which is worth ~8% of bandwidth
+// over eight workgroups reading one head each.  With fewer kv heads than wavefronts, the wavefronts of a
+// head interleave 16-token tiles and are merged through LDS at the end.
+//
+// Per tile and wavefront:
+//   global -> registers   coalesced 16-byte loads, each instruction reads whole cache rows (head_dim 128: four
+//                          256-byte bf16 rows or eight 128-byte fp8 rows); a tile's loads are in flight while
+//                          the previous tile is computed.  Rows
+//                          past the end of the chunk are clamped to the last valid row, so every load is in
+//                          bounds and finite.
+//   registers -> LDS       a private scratch per wavefront (64 x head_dim bytes), XOR-swizzled in 16-byte chunks; fp8 is
+//                          dequantised to the q dtype on the way (K as round(k8*scale), V exactly)
+//   S^T = K Q^T            head_dim/32 x v_mfma_f32_16x16x32 (A = K rows read back as ds_read_b128, B = Q^T kept in
+//                          registers); lane (h, a) then holds the logits of head h for tokens 4a..4a+3
+//   online softmax         fp32, running max shared by the four lane groups of a head
+//   O^T += V^T P^T         head_dim/16 x v_mfma_f32_16x16x16 (A = V^T through the LDS transpose read
+//                          ds_read_b64_tr_b16, B = P^T taken straight from the softmax registers)
+#pragma once
+
+#include "fdk_device.h"
+
+namespace fdk {
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+enum PageMode { PM_TILE = 0, PM_LOAD = 1, PM_LANE = 2, PM_LANE_DIV = 3 };
+template <bool B> struct BoolTag { static constexpr bool value = B; };
+
+constexpr int kTile = 16;                 // tokens per tile
+
+template <int QDT> struct Mma;
+template <> struct Mma<FDK_BF16> {
+    static __device__ __forceinline__ f32x4_t qk(uint4 a, uint4 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t pv(uint2 a, uint2 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint2 read_tr(const char* p) {
+        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4_t, p)));
+    }
+};
+template <> struct Mma<FDK_FP16> {
+    static __device__ __forceinline__ f32x4_t qk(uint4 a, uint4 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t pv(uint2 a, uint2 b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint2 read_tr(const char* p) {
+        return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4_t, p)));
+    }
+};
+
+// byte offset of 16-byte chunk `c` of row `r` inside a staged tile of 16 rows x RB bytes (RB = 2 D >= 128)
+template <int RB> __device__ __forceinline__ int k_off(int r, int c) { return r * RB + ((c ^ (r & 7)) << 4); }
+template <int RB> __device__ __forceinline__ int v_off(int r, int c) { return r * RB + ((c ^ ((r & 3) << 1)) << 4); }
+
+template <bool FP8, int D>
+struct Regs {                                  // one tile in registers, as loaded
+    static constexpr int LPR = D * (FP8 ? 1 : 2) / 16;   // lanes (16-byte pieces) per cache row
+    static constexpr int RPL = 64 / LPR;                 // rows per load instruction
+    static constexpr int NJ = kTile / RPL;               // load instructions per tensor and tile
+    uint32_t k[NJ][4];
+    uint32_t v[NJ][4];
+};
+
+__device__ __forceinline__ void put(uint32_t (&dst)[4], const uint4 x) {
+    dst[0] = x.x;
+    dst[1] = x.y;
+    dst[2] = x.z;
+    dst[3] = x.w;
+}
+__device__ __forceinline__ uint4 get(const uint32_t (&src)[4]) { return make_uint4(src[0], src[1], src[2], src[3]); }
+
+template <int QDT, bool FP8, int PM, int NBUF, int D>
+__global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) {
+    using M = Mma<QDT>;
+    using P2 = Pack2<QDT>;
+    using R = Regs<FP8, D>;
+    constexpr int NJ = R::NJ;
+    constexpr int LPR = R::LPR;                // lanes per cache row
+    constexpr int RPL = R::RPL;                // rows per load instruction
+    constexpr int ES = FP8 ? 1 : 2;
+    constexpr int RB = 2 * D;                  // bytes of a staged (16-bit) row
+    constexpr int KS = D / 32;                 // k-steps of the QK product
+    constexpr int DB = D / 16;                 // 16-column blocks of the output
+    constexpr int kScratch = 2 * kTile * RB;   // LDS bytes per wavefront: K tile + V tile; also 16 fp32 output rows
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];      // [nw][kScratch] then m[nw][16], l[nw][16]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int a = lane >> 4;                   // lane group: MFMA k-group / token group
+    const int c = lane & 15;                   // MFMA row/column index
+    const int lrow = lane / LPR;               // row of this lane within a load
+    const int lpiece = lane % LPR;             // 16-byte piece of the row
+
+    const int nw = blockDim.x >> 6;
+    const int nh = p.hg_per_wg;                // kv heads per workgroup
+    const int ti_n = nw / nh;                  // wavefronts interleaving the tiles of one kv head
+    const int hl = wave % nh;
+    const int tix = wave / nh;
+    float* sm_m = reinterpret_cast<float*>(lds + nw * kScratch);
+    float* sm_l = sm_m + nw * 16;
+
+    int* const s_next = reinterpret_cast<int*>(sm_l + nw * 16);     // next work item (persistent mode)
+
+    // ---- one work item: (sequence, split, kv-head block, q-head tile) ------------------------------------------
+    auto run_item = [&](int wg) {
+    const int ht = wg % p.head_tiles;
+    wg /= p.head_tiles;
+    const int hgb = wg % p.hg_blocks;
+    wg /= p.hg_blocks;
+    const int split = wg % p.num_splits;
+    const int b = wg / p.num_splits;
+    const int kvh = hgb * nh + hl;
+    const int head0 = kvh * p.group + ht * 16;
+    const int heads_here = min(16, p.group - ht * 16);
+
+    // Issue everything that does not depend on kv_len first, so that the dependent chain before the first K/V
+    // load is as short as possible: Q^T (the B operand of S^T = K Q^T: lane (h = c, a) holds
+    // q[h][32 ks + 8 a .. +7]; columns past the group repeat its last head - their results are never stored,
+    // and nothing waits for a select) and, speculatively, the page of this wave's first tile (any table column
+    // may be read; the value is used only if the tile exists).
+    uint4 qb[KS];
+    {
+        const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
+                             (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+    }
+    const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
+    const int c_start = split * p.chunk;
+    int first_pg = 0;
+    if (PM == PM_TILE) first_pg = tbl[min(c_start + tix * kTile, p.max_tokens - 1) >> p.page_shift];
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
+    if (c_start >= kv_len) {
+        if (p.direct && tix == 0) {   // kv_len == 0 with a single split: defined result, no combine follows
+            for (int idx = lane; idx < heads_here * D; idx += 64) {
+                const int g = idx / D, d = idx % D;
+                const int64_t ob = (int64_t)b * p.out_sb + (int64_t)(head0 + g) * p.out_sh;
+                store_out(p.out, ob + d, 0.f, p.out_dtype);
+                if (d == 0) {
+                    if (p.lse) p.lse[(int64_t)b * p.lse_sb + head0 + g] = -INFINITY;
+                    if (p.pack_lse) store_out(p.out, ob + D, -INFINITY, p.out_dtype);
+                }
+            }
+        }
+        return;
+    }
+    const int c_end = min(c_start + p.chunk, kv_len);
+
+    float kscale = 1.f, vscale = 1.f;
+    if (FP8) {
+        if (p.k_scale) kscale = p.k_scale[kvh];
+        if (p.v_scale) vscale = p.v_scale[kvh];
+    }
+    const bool softcap = p.soft_cap > 0.f;
+    const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
+
+    const char* kbase = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES + lpiece * 16;
+    const char* vbase = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES + lpiece * 16;
+    const int pmask = p.page_size - 1;
+    char* my_lds = lds + wave * kScratch;
+    char* lds_k = my_lds;
+    char* lds_v = my_lds + kScratch / 2;
+
+    struct PageIds { int32_t pg[PM == PM_TILE ? 1 : NJ]; };
+
+    auto pages_of = [&](int t, PageIds& pi) {
+        const int tok0 = c_start + t * kTile;
+        if (PM == PM_TILE) {
+            pi.pg[0] = tbl[tok0 >> p.page_shift];
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                int n = tok0 + j * RPL;
+                if (PM >= PM_LANE) n += lrow;
+                n = min(n, c_end - 1);
+                pi.pg[PM == PM_TILE ? 0 : j] = tbl[PM == PM_LANE_DIV ? n / p.page_size : n >> p.page_shift];
+            }
+        }
+    };
+    auto issue = [&](int t, const PageIds& pi, R& rg) {
+        const int tok0 = c_start + t * kTile;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int n = min(tok0 + j * RPL + lrow, c_end - 1);      // clamp: always a valid, finite row
+            const int slot = PM == PM_LANE_DIV ? n % p.page_size : (n & pmask);
+            const int64_t pg = pi.pg[PM == PM_TILE ? 0 : j];
+            put(rg.k[j], *reinterpret_cast<const uint4*>(kbase + (pg * p.k_sp + (int64_t)slot * p.k_st) * ES));
+            put(rg.v[j], *reinterpret_cast<const uint4*>(vbase + (pg * p.v_sp + (int64_t)slot * p.v_st) * ES));
+        }
+    };
+
+    // PM_TILE: a tile never leaves its page, so a load address is (page base + first slot of the tile), which
+    // is wave-uniform, plus a per-lane byte offset that is the same for every full tile.
+    uint32_t koff[NJ], voff[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        koff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.k_st) * ES + lpiece * 16);
+        voff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.v_st) * ES + lpiece * 16);
+    }
+    const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;   // wave-uniform
+    const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
+    auto issue_full = [&](int t, const PageIds& pi, R& rg) {
+        if (PM == PM_TILE) {
+            const int tok0 = c_start + t * kTile;
+            const int64_t pg = pi.pg[0];
+            const int slot0 = tok0 & pmask;
+            const char* kp = kplane + (pg * p.k_sp + (int64_t)slot0 * p.k_st) * ES;
+            const char* vp = vplane + (pg * p.v_sp + (int64_t)slot0 * p.v_st) * ES;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) put(rg.k[j], *reinterpret_cast<const uint4*>(kp + koff[j]));
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) put(rg.v[j], *reinterpret_cast<const uint4*>(vp + voff[j]));
+        } else {
+            issue(t, pi, rg);
+        }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;       // for head c; l_run is this lane group's share of the sum
+    f32x4_t acc[DB];                             // acc[db][i] = O[h = c][16 db + 4 a + i]
+#pragma unroll
+    for (int db = 0; db < DB; ++db) acc[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // registers -> LDS (16-bit elements, swizzled).  Once staged, the registers are free for the next tile's loads.
+    auto stage = [&](const R& rg) {
+        if (FP8) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int r = j * RPL + lrow;
+                uint32_t ko[8], vo[8];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    // K: (k8 * scale) rounded to the q dtype, i.e. the dequantised cache the reference decodes
+                    const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], false);
+                    const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], true);
+                    ko[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
+                    ko[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
+                    // V: exact conversion; its scale multiplies the output once at the end
+                    const f32x2_t v01 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.v[j][w], false);
+                    const f32x2_t v23 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.v[j][w], true);
+                    vo[2 * w] = P2::pack(v01.x, v01.y);
+                    vo[2 * w + 1] = P2::pack(v23.x, v23.y);
+                }
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int ch = 2 * lpiece + half;
+                    *reinterpret_cast<uint4*>(lds_k + k_off<RB>(r, ch)) =
+                        make_uint4(ko[4 * half], ko[4 * half + 1], ko[4 * half + 2], ko[4 * half + 3]);
+                    *reinterpret_cast<uint4*>(lds_v + v_off<RB>(r, ch)) =
+                        make_uint4(vo[4 * half], vo[4 * half + 1], vo[4 * half + 2], vo[4 * half + 3]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int r = j * RPL + lrow;
+                *reinterpret_cast<uint4*>(lds_k + k_off<RB>(r, lpiece)) = get(rg.k[j]);
+                *reinterpret_cast<uint4*>(lds_v + v_off<RB>(r, lpiece)) = get(rg.v[j]);
+            }
+        }
+    };
+
+    auto compute = [&](int t, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const int tok0 = c_start + t * kTile;
+        // ---- S^T[token][head] = K Q^T ----
+        f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4 ka = *reinterpret_cast<const uint4*>(lds_k + k_off<RB>(c, 4 * ks + a));
+            s = M::qk(ka, qb[ks], s);
+        }
+        // ---- online softmax for head c over tokens 4a .. 4a+3 of this tile ----
+        float sv[4] = {s.x, s.y, s.z, s.w};
+        if (softcap) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * p.sm_scale, p.soft_cap, inv_cap) * kLog2e;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sv[i] *= p.scale_log2;
+        }
+        if (MASKED) {                         // the partial last tile of the chunk
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (tok0 + 4 * a + i >= c_end) sv[i] = -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));          // finite: token tok0 is valid
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = fast_exp2(m_run - m_new);
+        float pr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pr[i] = fast_exp2(sv[i] - m_new);
+        l_run = l_run * alpha + (pr[0] + pr[1]) + (pr[2] + pr[3]);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+        }
+        m_run = m_new;
+        // P^T as B operand: lane (h = c, a) supplies p for tokens 4a..4a+3, rounded to the cache dtype as the
+        // reference does before its second dot (flash_decode.py:230)
+        const uint2 pb = make_uint2(P2::pack(pr[0], pr[1]), P2::pack(pr[2], pr[3]));
+        // ---- O^T[d][head] += V^T P^T ----
+        const int k4 = c >> 2, cc = c & 3;
+        const int vrow = 4 * a + k4;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const uint2 va = M::read_tr(lds_v + v_off<RB>(vrow, 2 * db + (cc >> 1)) + (cc & 1) * 8);
+            acc[db] = M::pv(va, pb, acc[db]);
+        }
+    };
+
+    // ---- pipeline over the full tiles: a tile is copied to LDS as soon as it has arrived, the next tile's
+    // loads are issued into the same registers, and the arithmetic on the staged tile overlaps them.  The
+    // partial last tile of the chunk goes to the wave whose turn it is.
+    const int n_full = (c_end - c_start) / kTile;
+    {
+        R rg;
+        PageIds pid;
+        int t = tix;
+        const int st = ti_n;
+        if (t < n_full) {
+            if (PM == PM_TILE) pid.pg[0] = first_pg; else pages_of(t, pid);
+            issue_full(t, pid, rg);
+            if (t + st < n_full) pages_of(t + st, pid);
+        }
+        if (NBUF == 1) {
+            // one register buffer: the next tile's loads go into the registers just staged
+            while (t < n_full) {
+                stage(rg);
+                const int tn = t + st;
+                if (tn < n_full) {
+                    issue_full(tn, pid, rg);
+                    if (tn + st < n_full) pages_of(tn + st, pid);
+                }
+                compute(t, BoolTag<false>());
+                t = tn;
+            }
+        } else {
+            // two register buffers: a second tile is requested before the first is staged.  The steady state
+            // always issues before it stages, so the waits on the older tile can be partial.
+            R rb;
+            while (t + 2 * st < n_full) {
+                issue_full(t + st, pid, rb);
+                pages_of(t + 2 * st, pid);
+                stage(rg);
+                compute(t, BoolTag<false>());
+                issue_full(t + 2 * st, pid, rg);
+                if (t + 3 * st < n_full) pages_of(t + 3 * st, pid);
+                stage(rb);
+                compute(t + st, BoolTag<false>());
+                t += 2 * st;
+            }
+            if (t + st < n_full) {
+                issue_full(t + st, pid, rb);
+                stage(rg);
+                compute(t, BoolTag<false>());
+                stage(rb);
+                compute(t + st, BoolTag<false>());
+            } else if (t < n_full) {
+                stage(rg);
+                compute(t, BoolTag<false>());
+            }
+        }
+        if (n_full * kTile < c_end - c_start && (n_full % ti_n) == tix) {
+            pages_of(n_full, pid);
+            issue(n_full, pid, rg);
+            stage(rg);
+            compute(n_full, BoolTag<true>());
+        }
+    }
+
+    // ---- merge: lane groups (sum of l), then the wavefronts that share a kv head through LDS --------------
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    float* my_o = reinterpret_cast<float*>(my_lds);          // [16 heads][D] fp32 = this wave's scratch
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+        *reinterpret_cast<float4*>(my_o + c * D + 16 * db + 4 * a) =
+            make_float4(acc[db].x, acc[db].y, acc[db].z, acc[db].w);
+    if (a == 0) {
+        sm_m[wave * 16 + c] = m_run;
+        sm_l[wave * 16 + c] = l_run;
+    }
+    if (ti_n > 1) __syncthreads();                           // ti_n == 1: a wave reads back only its own rows
+    const float* all_o = reinterpret_cast<const float*>(lds);
+    // wave w writes the rows of kv head (w % nh), sharing the work with the waves of the same head
+    for (int idx = tix * 64 + lane; idx < heads_here * D; idx += ti_n * 64) {
+        const int g = idx / D, d = idx % D;
+        float mx = -INFINITY;
+        for (int t = 0; t < ti_n; ++t) mx = fmaxf(mx, sm_m[(hl + nh * t) * 16 + g]);
+        float o = 0.f, l = 0.f;
+        for (int t = 0; t < ti_n; ++t) {
+            const int w = hl + nh * t;
+            const float sc = fast_exp2(sm_m[w * 16 + g] - mx);     // mx is finite: the chunk holds >= 1 token
+            o += all_o[w * (kScratch / 4) + g * D + d] * sc;
+            l += sm_l[w * 16 + g] * sc;
+        }
+        const float res = o * vscale / l;
+        const int hq = head0 + g;
+        const float lse_nat = (mx + fast_log2(l)) * kLn2;
+        if (p.direct) {
+            const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh;
+            store_out(p.out, ob + d, res, p.out_dtype);
+            if (d == 0) {
+                if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
+                if (p.pack_lse) store_out(p.out, ob + D, lse_nat, p.out_dtype);
+            }
+        } else {
+            const int64_t row = ((int64_t)b * p.hq + hq) * p.num_splits + split;
+            p.part_o[row * D + d] = res;
+            if (d == 0) p.part_lse[row] = lse_nat;
+        }
+    }
+
+    };   // run_item
+
+    // ---- work distribution: one item per workgroup, or (persistent) a fixed set of workgroups that pull items
+    // from a queue: counters[0] is its head, counters[1] counts finished workgroups; the last one to finish
+    // puts both back to zero.  The first item of every workgroup is its own index.
+    int item = blockIdx.x;
+    while (item < p.total_items) {
+        run_item(item);
+        if (!p.persistent) return;
+        __syncthreads();
+        if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
+        __syncthreads();
+        item = s_next[0];
+    }
+    if (threadIdx.x == 0) {
+        const int done = atomicAdd(p.counters + 1, 1);
+        if (done == (int)gridDim.x - 1) {
+            atomicExch(p.counters, 0);
+            atomicExch(p.counters + 1, 0);
+        }
+    }
+}
+
+template <int QDT, bool FP8, int D>
+int launch_pm(const SplitParams& p_in, hipStream_t stream) {
+    constexpr int kScratch = 4 * kTile * D;
+    SplitParams p = p_in;
+    p.head_tiles = (p.group + 15) / 16;
+    if (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) p.hg_per_wg = 1;
+    p.hg_blocks = p.hkv / p.hg_per_wg;
+    const int nw = p.hg_per_wg > 4 ? p.hg_per_wg : 4;
+    const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float)) + 16;
+    constexpr int RPL = Regs<FP8, D>::RPL;
+    int pm;
+    if (p.page_shift < 0) pm = PM_LANE_DIV;
+    else if (p.page_size % kTile == 0) pm = PM_TILE;
+    else if (p.page_size % RPL == 0) pm = PM_LOAD;
+    else pm = PM_LANE;
+    p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
+    // Persistent mode (work queue) whenever the KV range is split and the caller provided counters: items of a
+    // ragged batch differ in length, and a queue keeps every compute unit busy until the end.
+    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
+    p.persistent = (p.counters != nullptr && !p.direct && p.total_items > resident) ? 1 : 0;
+    const dim3 grid((unsigned)(p.persistent ? resident : p.total_items));
+    const dim3 block(64 * nw);
+    // Two register buffers per wavefront, except for the widest rows where they would not leave room for two
+    // workgroups per compute unit.
+    constexpr int NBUF = D > 128 ? 1 : 2;
+#define FDK_MFMA_LAUNCH(PMV) \
+    hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NBUF, D>), grid, block, lds_bytes, stream, p)
+    switch (pm) {
+        case PM_TILE: FDK_MFMA_LAUNCH(PM_TILE); break;
+        case PM_LOAD: FDK_MFMA_LAUNCH(PM_LOAD); break;
+        case PM_LANE: FDK_MFMA_LAUNCH(PM_LANE); break;
+        default: FDK_MFMA_LAUNCH(PM_LANE_DIV); break;
+    }
+#undef FDK_MFMA_LAUNCH
+    return (int)hipGetLastError();
+}
+
+
+template <int D>
+int launch_mfma_d(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    const bool fp8 = kv_dtype == FDK_FP8_E4M3;
+    if (q_dtype == FDK_BF16)
+        return fp8 ? launch_pm<FDK_BF16, true, D>(p, stream) : launch_pm<FDK_BF16, false, D>(p, stream);
+    return fp8 ? launch_pm<FDK_FP16, true, D>(p, stream) : launch_pm<FDK_FP16, false, D>(p, stream);
+}
+
+}  // namespace
+
+}  // namespace fdk

@@ -20,7 +20,8 @@ int valu_heads_per_wg(int group) {
     return 8;
 }
 
-bool valu_supported(int q_dtype, int kv_dtype, int /*group*/) {
+bool valu_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim) {
+    if (head_dim != kHeadDim) return false;
     if (q_dtype != FDK_BF16 && q_dtype != FDK_FP16) return false;
     return kv_dtype == q_dtype || kv_dtype == FDK_FP8_E4M3;
 }
