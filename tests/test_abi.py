@@ -175,27 +175,47 @@ def test_plan_scales_splits_with_occupancy():
     p = _plan(_args())                                    # 256 (sequence, kv head) units on 256 CUs
     assert p.num_splits == 1 and p.chunk_tokens >= 4096   # they fill the device: one pass, no combine
     assert p.algo == _lib.FDK_ALGO_MFMA
-    # fewer sequences: the KV range is split, chunks are multiples of 64 tokens and cover the range
+    # fewer sequences, short context: chunk mode - chunks are multiples of 64 tokens and cover the range
     p4 = _plan(_args(batch=4))
-    assert p4.num_splits > 1 and p4.chunk_tokens % 64 == 0
+    assert p4.balanced == 0 and p4.num_splits > 1 and p4.chunk_tokens % 64 == 0
     assert p4.num_splits * p4.chunk_tokens >= 4096 > (p4.num_splits - 1) * p4.chunk_tokens
-    # few units, long context -> many splits; chunks of a long context are never shorter than 512 tokens
+    # few units, long context: balanced mode - two workgroups per compute unit share the KV ranges of the whole
+    # batch, each gets a long share, and the workspace holds (shares + batch) slots per head block
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
                          q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
-    assert p_long.num_splits >= p4.num_splits and p_long.chunk_tokens >= 512 > p4.chunk_tokens
-    # a short context is latency-bound: it is split down to chunks of 64 tokens, never finer
+    assert p_long.balanced == 1 and p_long.workgroups == 512 and p_long.chunk_tokens >= 512
+    units = 8 // p_long.kv_heads_per_wg
+    shares = p_long.workgroups // units
+    rows = (shares + 4) * units * p_long.kv_heads_per_wg * 8           # group = 8 heads per tile
+    assert p_long.num_splits * 4 * 64 >= rows > (p_long.num_splits - 1) * 4 * 64
+    assert shares * p_long.chunk_tokens >= 4 * 131072                   # the shares cover every sequence
+    # a short context is latency-bound: chunk mode, split down to chunks of 64 tokens, never finer
     p_short = _plan(_args(batch=1, max_pages=8, table_stride_b=8))
-    assert p_short.num_splits == 2 and p_short.chunk_tokens == 64
-    p_one = _plan(_args(batch=1, max_pages=4, table_stride_b=4))
-    assert p_one.num_splits == 1 and p_one.chunk_tokens == 64
-    # the host's bound on kv_len drives the split, not the table width
+    assert p_short.balanced == 0 and p_short.num_splits == 2 and p_short.chunk_tokens == 64
+    p_one = _plan(_args(batch=1, max_pages=4, table_stride_b=4))      # 64 tokens: nothing to split
+    assert p_one.num_splits == 1 and p_one.balanced == 0
+    # the host's bound on kv_len drives the plan, not the table width
     p_hint = _plan(_args(batch=4, max_pages=2048, table_stride_b=2048, max_kv_len=4096))
-    assert (p_hint.num_splits, p_hint.chunk_tokens) == (p4.num_splits, p4.chunk_tokens)
-    # a forced split count is honoured and covers the whole range
+    assert (p_hint.num_splits, p_hint.workgroups, p_hint.chunk_tokens) == (p4.num_splits, p4.workgroups, p4.chunk_tokens)
+    # a forced split count is honoured in chunk mode: chunks are multiples of 64 tokens and cover the range
     p_forced = _plan(_args(num_splits=32))
-    assert p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
-    # fewer compute units -> no more splits than with many
+    assert p_forced.balanced == 0 and p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
+    p_f4 = _plan(_args(batch=4, num_splits=5))
+    assert p_f4.balanced == 0 and p_f4.chunk_tokens % 64 == 0
+    assert 5 * p_f4.chunk_tokens >= 4096 > 4 * p_f4.chunk_tokens
+    # the vector path splits in chunk mode
+    p_v = _plan(_args(batch=4, algo=_lib.FDK_ALGO_VALU))
+    assert p_v.balanced == 0 and p_v.num_splits > 1
+    assert p_v.num_splits * p_v.chunk_tokens >= 4096 > (p_v.num_splits - 1) * p_v.chunk_tokens
+    # fewer compute units -> no more splits / workgroups than with many
     assert _plan(_args(batch=4), cus=64).num_splits <= p4.num_splits
+    assert _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048, q_stride_b=64 * 128,
+                       out_stride_b=64 * 128, lse_stride_b=64), cus=64).workgroups <= p_long.workgroups
+    # very large batches stay in chunk mode (every wavefront would have to scan kv_lens)
+    assert _plan(_args(batch=600, num_q_heads=1, num_kv_heads=1, q_stride_b=128, out_stride_b=128, lse_stride_b=1,
+                       max_pages=4096, table_stride_b=4096), cus=1024).balanced == 0
+    assert _plan(_args(batch=500, num_q_heads=1, num_kv_heads=1, q_stride_b=128, out_stride_b=128, lse_stride_b=1,
+                       max_pages=4096, table_stride_b=4096), cus=1024).balanced == 1
     # the vector path can be forced
     assert _plan(_args(algo=_lib.FDK_ALGO_VALU)).algo == _lib.FDK_ALGO_VALU
 

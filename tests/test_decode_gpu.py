@@ -411,6 +411,97 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
     torch.testing.assert_close(final2.double().cpu(), want, atol=4e-3, rtol=1e-2)
 
 
+# ---- balanced mode: the kernel cuts the batch's KV ranges into equal shares from kv_lens ---------------------------
+BALANCED_CASES = {
+    # name: (kv_lens, (Hq, Hkv), page, head_dim, fp8)
+    "one_long_two_short": ([40000, 0, 777], (8, 1), 16, 128, False),
+    "short_first": ([1, 39999, 64, 65], (8, 1), 16, 128, False),
+    "all_heads_two_per_wg": ([30000, 12345, 5, 0, 20000], (32, 8), 16, 128, False),
+    "group16_p64": ([50000, 3, 17000], (16, 1), 64, 128, False),
+    "group24_two_tiles": ([40000, 30000], (24, 1), 16, 128, False),
+    "page1": ([9000, 40000, 1], (8, 2), 1, 128, False),
+    "fp8_d128": ([33000, 100, 8000], (16, 2), 16, 128, True),
+    "d64": ([33000, 100, 8000], (8, 2), 16, 64, False),
+    "d256": ([33000, 100, 8000], (8, 2), 16, 256, False),
+    "odd_page24": ([40000, 4097, 23], (8, 1), 24, 128, False),
+}
+
+
+@pytest.mark.parametrize("name", list(BALANCED_CASES))
+def test_balanced_mode_ragged_batches(cuda_device, name):
+    lens, (hq, hkv), page, d, fp8 = BALANCED_CASES[name]
+    print(f"case balanced {name}", flush=True)
+    g = torch.Generator().manual_seed(hash(name) & 0xFFFF)
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 3
+    width = max(pages) + 2
+    q = torch.randn(len(lens), hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((len(lens), width), 2 ** 31 - 1, dtype=torch.int32)      # poisoned beyond each sequence
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    ks = vs = None
+    ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks), ofp8.dequant_per_head(v, vs))
+    scale = d ** -0.5
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens))
+    assert plan.balanced and plan.workgroups > 0, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=max(lens), k_scale=ks, v_scale=vs)
+    # chunk mode on the same inputs (a forced split count)
+    out_c, lse_c = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=max(lens), k_scale=ks, v_scale=vs,
+                                    kv_split=7)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    empty = [i for i, n in enumerate(lens) if n == 0]
+    for o, l, tag in ((out, lse, "balanced"), (out_c, lse_c, "chunks")):
+        if empty:
+            assert (o[empty] == 0).all() and torch.isinf(l[empty]).all() and (l[empty] < 0).all()
+        _check(o[live], l[live], q[live], k, v, table[live], [lens[i] for i in live], scale, ref_kv=ref_kv,
+               tag=f"{name} {tag}")
+    torch.testing.assert_close(out.float(), out_c.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse[live], lse_c[live], atol=1e-4, rtol=0)
+
+
+def test_balanced_mode_many_sequences(cuda_device):
+    # more than 64 sequences: the partition scan runs over several 64-lane chunks; includes empty sequences
+    g = torch.Generator().manual_seed(77)
+    b, hq, hkv, d, page = 150, 8, 1, 128, 16
+    lens = torch.randint(0, 6001, (b,), generator=g).tolist()
+    for i in (0, 63, 64, 65, 127, 128, 149):
+        lens[i] = 0
+    lens[1], lens[66], lens[148] = 6000, 1, 5999
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 1
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.zeros((b, max(pages)), dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=6000)
+    assert plan.balanced, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=6000)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    empty = [i for i, n in enumerate(lens) if n == 0]
+    assert (out[empty] == 0).all() and (lse[empty] == float("-inf")).all()
+    _check(out[live], lse[live], q[live], k, v, table[live], [lens[i] for i in live], d ** -0.5, tag="balanced b150")
+
+
 @pytest.mark.parametrize("page", [6, 24])
 @pytest.mark.parametrize("algo", ["valu", "mfma"])
 def test_page_sizes_that_are_not_powers_of_two(cuda_device, page, algo):

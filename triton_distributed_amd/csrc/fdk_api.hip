@@ -61,6 +61,8 @@ constexpr int kChunkAlign = 64;     // split boundaries fall on multiples of 64 
 constexpr int kMinChunk = 64;       // shortest chunk (short contexts: latency matters more than the partials)
 constexpr int kMaxMinChunk = 512;   // long contexts are never split finer than this
 constexpr int kMaxSplits = 1024;
+constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
+constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
 
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
     if (!a) return fail(FDK_ENULL, "args is null");
@@ -163,6 +165,9 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // The shortest chunk grows with the context (max_len / 64, between kMinChunk and kMaxMinChunk tokens):
     // a short context is latency-bound and gains from every extra split, a long one pays for each partial
     // row it writes and re-reads.
+    int64_t min_chunk = cdiv64(cdiv64(max_len, 64), kChunkAlign) * kChunkAlign;
+    if (min_chunk < kMinChunk) min_chunk = kMinChunk;
+    if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
     int64_t splits;
     if (a->num_splits > 0) {
         splits = a->num_splits;
@@ -170,12 +175,37 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         splits = 1;
     } else {
         splits = cdiv64(2 * (int64_t)num_cus, units);
-        int64_t min_chunk = cdiv64(cdiv64(max_len, 64), kChunkAlign) * kChunkAlign;
-        if (min_chunk < kMinChunk) min_chunk = kMinChunk;
-        if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
         const int64_t cap = cdiv64(max_len, min_chunk);
         if (splits > cap) splits = cap;
         if (splits < 1) splits = 1;
+    }
+    memset(plan, 0, sizeof(*plan));
+    plan->algo = algo;
+    plan->kv_heads_per_wg = kv_heads_per_wg;
+
+    // Balanced mode replaces the per-sequence chunks whenever the matrix-core path would split on its own
+    // account: the kernel cuts the KV ranges of the whole batch, as kv_lens gives them, into equal shares, so
+    // that a ragged batch loads every workgroup alike.  The workspace then holds (shares + batch) slots of
+    // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
+    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && splits > 1 && batch <= kMaxBalancedBatch) {
+        const int64_t gran = fdk::kBalanceGranule;
+        const int64_t columns = (int64_t)batch * cdiv64(max_len, gran);      // granules of all sequences, at most
+        int64_t shares = columns / (min_chunk / gran);
+        const int64_t most = 2 * (int64_t)num_cus / units_per_seq;           // two workgroups per compute unit
+        if (shares > most) shares = most;
+        if (shares < 1) shares = 1;
+        const int64_t share_tokens = cdiv64(columns, shares) * gran;
+        // Deriving the partition costs every workgroup a pass over kv_lens before its first load: worth it
+        // only when a share is long enough to hide that.
+        if (share_tokens >= kMinBalancedShare) {
+            const int64_t rows_per_slot = (int64_t)kv_heads_per_wg * (group < 16 ? group : 16);
+            const int64_t rows = (shares + batch) * units_per_seq * rows_per_slot;
+            plan->balanced = 1;
+            plan->workgroups = (int32_t)(shares * units_per_seq);
+            plan->num_splits = (int32_t)cdiv64(rows, (int64_t)batch * a->num_q_heads);
+            plan->chunk_tokens = (int32_t)(cdiv64(share_tokens, kChunkAlign) * kChunkAlign);
+            return FDK_OK;
+        }
     }
     int64_t chunk = cdiv64(cdiv64(max_len, splits), kChunkAlign) * kChunkAlign;
     if (a->num_splits <= 0) splits = cdiv64(max_len, chunk);   // drop splits that would always be empty
@@ -185,14 +215,13 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     }
     plan->num_splits = (int32_t)splits;
     plan->chunk_tokens = (int32_t)chunk;
-    plan->algo = algo;
-    plan->reserved = kv_heads_per_wg;
     return FDK_OK;
 }
 
-int head_tiles_of(const fdk_decode_args* a) {
+// q-head tiles per kv head, as the resolved algorithm's kernel counts them
+int head_tiles_of(const fdk_decode_args* a, int algo) {
     const int group = a->num_q_heads / a->num_kv_heads;
-    const int hpw = fdk::valu_heads_per_wg(group);
+    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group) : fdk::valu_heads_per_wg(group);
     return (group + hpw - 1) / hpw;
 }
 
@@ -208,7 +237,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     const int S = r->plan.num_splits;
     const bool direct = direct_ok && S == 1;
     const int64_t rows = (int64_t)a->batch * a->num_q_heads;
-    if ((int64_t)a->batch * S * a->num_kv_heads * head_tiles_of(a) > INT32_MAX)
+    if ((int64_t)a->batch * S * a->num_kv_heads * head_tiles_of(a, r->plan.algo) > INT32_MAX)
         return fail(FDK_ESHAPE, "grid too large");
     float* part_o = nullptr;
     float* part_lse = nullptr;
@@ -242,8 +271,12 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
     sp.num_splits = S; sp.chunk = r->plan.chunk_tokens;
     sp.max_tokens = (int32_t)((int64_t)a->max_pages * a->page_size);
-    sp.head_tiles = head_tiles_of(a);
-    sp.hg_per_wg = r->plan.reserved;
+    sp.head_tiles = head_tiles_of(a, r->plan.algo);
+    sp.hg_per_wg = r->plan.kv_heads_per_wg;
+    sp.balanced = r->plan.balanced;
+    sp.workgroups = r->plan.workgroups;
+    sp.heads_per_tile = sp.group < 16 ? sp.group : 16;
+    sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
@@ -260,6 +293,10 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     cp.num_splits = S; cp.chunk = r->plan.chunk_tokens;
     cp.max_tokens = sp.max_tokens;
     cp.out_dtype = a->out_dtype; cp.pack_lse = sp.pack_lse;
+    cp.balanced = sp.balanced; cp.workgroups = sp.workgroups;
+    cp.group = sp.group; cp.kv_heads_per_wg = sp.hg_per_wg; cp.head_tiles = sp.head_tiles;
+    cp.hg_blocks = a->num_kv_heads / (sp.hg_per_wg > 0 ? sp.hg_per_wg : 1);
+    cp.rows_per_slot = sp.rows_per_slot; cp.heads_per_tile = sp.heads_per_tile;
     return FDK_OK;
 }
 
@@ -323,7 +360,7 @@ int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
     if (rc) return rc;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     // work-queue form of the split kernel (matrix-core path only)
-    const bool queued = !r.sp.direct && args->counters != nullptr && r.plan.algo == FDK_ALGO_MFMA;
+    const bool queued = !r.sp.direct && !r.sp.balanced && args->counters != nullptr && r.plan.algo == FDK_ALGO_MFMA;
     if (queued) {
         if (reinterpret_cast<uintptr_t>(args->counters) & 3u) return fail(FDK_EALIGN, "counters not 4-byte aligned");
         if (args->counters_len < fdk_counters_len(args))

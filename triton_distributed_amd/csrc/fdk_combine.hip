@@ -34,6 +34,64 @@ template <> struct Vec<4> {
     }
 };
 
+// Where the partial rows of output row (b, h) are: `live` rows, the s-th at o[s * o_step] / lse[s * lse_step].
+struct PartRows {
+    const float* o;
+    const float* lse;
+    int64_t o_step;
+    int lse_step;
+    int live;
+};
+
+template <int D>
+__device__ __forceinline__ PartRows locate_rows(const CombineParams& p, int b, int h) {
+    PartRows r;
+    if (!p.balanced) {
+        // chunk mode: split c holds tokens [c*chunk, ...) - the split kernel wrote exactly the live ones
+        const int kv_len = min(p.kv_lens[b], p.max_tokens);
+        const int64_t row = (int64_t)b * p.hq + h;
+        r.live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
+        r.o = p.part_o + row * p.num_splits * D;
+        r.lse = p.part_lse + row * p.num_splits;
+        r.o_step = D;
+        r.lse_step = 1;
+        return r;
+    }
+    // balanced mode: redo the split kernel's partition.  The sequences, in granules laid end to end, are cut
+    // into `shares` equal parts (the first `rem` one granule longer); sequence b spans granules
+    // [before, before + mine); the piece of share wc for unit u is in slot (wc + b) * units + u.
+    const int lane = threadIdx.x & 63;
+    const int units = p.hg_blocks * p.head_tiles;
+    int total = 0, before = 0;
+    for (int b0 = 0; b0 < p.batch; b0 += 64) {
+        const int bb = b0 + lane;
+        const int g = bb < p.batch ? (max(min(p.kv_lens[bb], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule : 0;
+        total += g;
+        before += bb < b ? g : 0;
+    }
+    total = wave_sum_i32(total);
+    before = wave_sum_i32(before);
+    const int mine = (max(min(p.kv_lens[b], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule;
+    const int kvh = h / p.group, hin = h % p.group;
+    const int u = (kvh / p.kv_heads_per_wg) * p.head_tiles + hin / 16;
+    const int row_in_slot = (kvh % p.kv_heads_per_wg) * p.heads_per_tile + hin % 16;
+    r.o_step = (int64_t)units * p.rows_per_slot * D;
+    r.lse_step = units * p.rows_per_slot;
+    r.live = 0;
+    r.o = p.part_o;
+    r.lse = p.part_lse;
+    if (mine == 0) return r;
+    const int shares = min(p.workgroups / units, total);
+    const int q = total / shares, rem = total % shares;
+    auto share_of = [&](int x) { return x < rem * (q + 1) ? x / (q + 1) : rem + (x - rem * (q + 1)) / q; };
+    const int wc_first = share_of(before), wc_last = share_of(before + mine - 1);
+    const int64_t row0 = ((int64_t)(wc_first + b) * units + u) * p.rows_per_slot + row_in_slot;
+    r.live = wc_last - wc_first + 1;
+    r.o = p.part_o + row0 * D;
+    r.lse = p.part_lse + row0;
+    return r;
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     constexpr int EPL = D / 64;
@@ -42,12 +100,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + wave;   // b * Hq + h
     if (row >= (int64_t)p.batch * p.hq) return;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
-    const int kv_len = min(p.kv_lens[b], p.max_tokens);
-    // live splits: chunk c holds tokens [c*chunk, ...) - the split kernel wrote exactly these
-    const int live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
-
-    const float* lse_row = p.part_lse + row * p.num_splits;
-    const float* o_row = p.part_o + row * p.num_splits * D + EPL * lane;
+    const PartRows pr = locate_rows<D>(p, b, h);
+    const int live = pr.live;
+    const float* lse_row = pr.lse;
+    const float* o_row = pr.o + EPL * lane;
 
     float m_run = -INFINITY, l_run = 0.f;
     float acc[EPL];
@@ -55,7 +111,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
     for (int s0 = 0; s0 < live; s0 += 64) {
         const int n = min(64, live - s0);
-        const float my = lane < n ? lse_row[s0 + lane] * kLog2e : -INFINITY;   // log2 units
+        const float my = lane < n ? lse_row[(s0 + lane) * pr.lse_step] * kLog2e : -INFINITY;   // log2 units
         const float m_blk = wave_max(my);
         const float m_new = fmaxf(m_run, m_blk);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -68,7 +124,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
         for (int s = 0; s < n; ++s) {
             const float ws = __shfl(w, s, 64);
             float o[EPL];
-            Vec<EPL>::load(o_row + (int64_t)(s0 + s) * D, o);
+            Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
 #pragma unroll
             for (int e = 0; e < EPL; ++e) acc[e] += ws * o[e];
         }
@@ -99,14 +155,14 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     const int wave = threadIdx.x >> 6;
     const int64_t row = blockIdx.x;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
-    const int kv_len = min(p.kv_lens[b], p.max_tokens);
-    const int live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
-    const float* lse_row = p.part_lse + row * p.num_splits;
-    const float* o_row = p.part_o + row * p.num_splits * D + EPL * lane;
+    const PartRows pr = locate_rows<D>(p, b, h);
+    const int live = pr.live;
+    const float* lse_row = pr.lse;
+    const float* o_row = pr.o + EPL * lane;
 
     float m = -INFINITY;
     for (int s0 = 0; s0 < live; s0 += 64) {
-        const float my = s0 + lane < live ? lse_row[s0 + lane] : -INFINITY;
+        const float my = s0 + lane < live ? lse_row[(s0 + lane) * pr.lse_step] : -INFINITY;
         m = fmaxf(m, wave_max(my));
     }
     m *= kLog2e;
@@ -116,13 +172,13 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
     for (int s0 = 0; s0 < live; s0 += 64) {
         const int n = min(64, live - s0);
-        const float w = lane < n ? fast_exp2(lse_row[s0 + lane] * kLog2e - m) : 0.f;
+        const float w = lane < n ? fast_exp2(lse_row[(s0 + lane) * pr.lse_step] * kLog2e - m) : 0.f;
         l += wave_sum(w);
 #pragma unroll 8
         for (int s = wave; s < n; s += kRowsPerWg) {
             const float ws = __shfl(w, s, 64);
             float o[EPL];
-            Vec<EPL>::load(o_row + (int64_t)(s0 + s) * D, o);
+            Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
 #pragma unroll
             for (int e = 0; e < EPL; ++e) acc[e] += ws * o[e];
         }
@@ -213,7 +269,9 @@ __global__ __launch_bounds__(256) void combine_ranks_kernel(const CombineRanksPa
 int launch_combine(const CombineParams& p, hipStream_t stream) {
     const int64_t rows = (int64_t)p.batch * p.hq;
     if (rows == 0) return 0;
-    const bool wide = p.num_splits > 8;
+    // pieces of a row: the split count, or in balanced mode about shares / sequences
+    const int units = p.hg_blocks * p.head_tiles;
+    const bool wide = (p.balanced ? p.workgroups / (units > 0 ? units : 1) / (p.batch > 0 ? p.batch : 1) + 1 : p.num_splits) > 8;
     const dim3 grid((unsigned)(wide ? rows : (rows + kRowsPerWg - 1) / kRowsPerWg));
 #define FDK_COMBINE_LAUNCH(DV)                                                                     \
     do {                                                                                           \

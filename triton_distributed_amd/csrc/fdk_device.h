@@ -10,6 +10,7 @@ namespace fdk {
 
 constexpr int kHeadDim = 128;       // head dimension of the vector path (the matrix-core path: 64, 128, 256)
 constexpr int kWaveSize = 64;
+constexpr int kBalanceGranule = 64;  // tokens per unit of the balanced partition (a multiple of the 16-token tile)
 constexpr int kWavesPerWg = 4;      // split kernels run 256-thread workgroups
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -43,6 +44,8 @@ struct SplitParams {
     int32_t pack_lse;
     int32_t direct;                 // 1: single split, write the final (out, lse) instead of partials
     int32_t persistent, total_items, num_cus;
+    int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
+    int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     float scale_log2;               // sm_scale * log2(e)
     float soft_cap;                 // > 0: on (applied to natural-unit logits)
     float sm_scale;
@@ -60,6 +63,9 @@ struct CombineParams {
     int32_t max_tokens;
     int32_t out_dtype;
     int32_t pack_lse;
+    // balanced mode (see the split kernel): where the pieces of a (sequence, head) row are
+    int32_t balanced, workgroups;
+    int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile;
 };
 
 struct CombineRanksParams {
@@ -115,6 +121,23 @@ __device__ __forceinline__ float group_sum(float x) {
     if (LANES >= 16) x += dpp_mov<0x140>(x);  // row_mirror
     return x;
 }
+
+// Inclusive prefix sum over the 64 lanes with DPP row shifts and row broadcasts (no LDS traffic).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_add_i32(int x) {
+    // lanes outside ROW_MASK and shifted-in positions contribute 0
+    return x + __builtin_amdgcn_update_dpp(0, x, CTRL, ROW_MASK, 0xF, ROW_MASK == 0xF);
+}
+__device__ __forceinline__ int wave_scan_i32(int x) {
+    x = dpp_add_i32<0x111, 0xF>(x);   // row_shr:1
+    x = dpp_add_i32<0x112, 0xF>(x);   // row_shr:2
+    x = dpp_add_i32<0x114, 0xF>(x);   // row_shr:4
+    x = dpp_add_i32<0x118, 0xF>(x);   // row_shr:8  -> scan within each row of 16
+    x = dpp_add_i32<0x142, 0xA>(x);   // row_bcast:15 into rows 1 and 3
+    x = dpp_add_i32<0x143, 0xC>(x);   // row_bcast:31 into rows 2 and 3
+    return x;
+}
+__device__ __forceinline__ int wave_sum_i32(int x) { return __builtin_amdgcn_readlane(wave_scan_i32(x), 63); }
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll

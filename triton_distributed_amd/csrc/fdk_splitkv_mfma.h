@@ -42,6 +42,7 @@ enum PageMode { PM_TILE = 0, PM_LOAD = 1, PM_LANE = 2, PM_LANE_DIV = 3 };
 template <bool B> struct BoolTag { static constexpr bool value = B; };
 
 constexpr int kTile = 16;                 // tokens per tile
+constexpr int kGranule = kBalanceGranule; // balanced mode: tokens per unit of the partition
 
 template <int QDT> struct Mma;
 template <> struct Mma<FDK_BF16> {
@@ -121,14 +122,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     int* const s_next = reinterpret_cast<int*>(sm_l + nw * 16);     // next work item (persistent mode)
 
-    // ---- one work item: (sequence, split, kv-head block, q-head tile) ------------------------------------------
-    auto run_item = [&](int wg) {
-    const int ht = wg % p.head_tiles;
-    wg /= p.head_tiles;
-    const int hgb = wg % p.hg_blocks;
-    wg /= p.hg_blocks;
-    const int split = wg % p.num_splits;
-    const int b = wg / p.num_splits;
+    // ---- one piece of work: tokens [c_start, min(c_limit, kv_len)) of sequence b for kv-head block hgb and q-head
+    // tile ht.  Partial results of head g of the tile go to row prow0 + g * prow_step of the workspace.
+    auto run_piece = [&](const int b, const int hgb, const int ht, const int c_start, const int c_limit,
+                         const int64_t prow0, const int prow_step) {
     const int kvh = hgb * nh + hl;
     const int head0 = kvh * p.group + ht * 16;
     const int heads_here = min(16, p.group - ht * 16);
@@ -146,7 +143,6 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
     }
     const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
-    const int c_start = split * p.chunk;
     int first_pg = 0;
     if (PM == PM_TILE) first_pg = tbl[min(c_start + tix * kTile, p.max_tokens - 1) >> p.page_shift];
     const int kv_len = min(p.kv_lens[b], p.max_tokens);
@@ -164,7 +160,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         }
         return;
     }
-    const int c_end = min(c_start + p.chunk, kv_len);
+    const int c_end = min(c_limit, kv_len);
 
     float kscale = 1.f, vscale = 1.f;
     if (FP8) {
@@ -211,12 +207,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     // PM_TILE: a tile never leaves its page, so a load address is (page base + first slot of the tile), which
     // is wave-uniform, plus a per-lane byte offset that is the same for every full tile.
-    uint32_t koff[NJ], voff[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        koff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.k_st) * ES + lpiece * 16);
-        voff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.v_st) * ES + lpiece * 16);
-    }
+    const uint32_t koff = (uint32_t)(((int64_t)lrow * p.k_st) * ES + lpiece * 16);   // per lane
+    const uint32_t voff = (uint32_t)(((int64_t)lrow * p.v_st) * ES + lpiece * 16);
+    const int64_t kstep = (int64_t)RPL * p.k_st * ES;                                 // per load, wave-uniform
+    const int64_t vstep = (int64_t)RPL * p.v_st * ES;
     const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;   // wave-uniform
     const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
     auto issue_full = [&](int t, const PageIds& pi, R& rg) {
@@ -227,9 +221,9 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const char* kp = kplane + (pg * p.k_sp + (int64_t)slot0 * p.k_st) * ES;
             const char* vp = vplane + (pg * p.v_sp + (int64_t)slot0 * p.v_st) * ES;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) put(rg.k[j], *reinterpret_cast<const uint4*>(kp + koff[j]));
+            for (int j = 0; j < NJ; ++j) put(rg.k[j], *reinterpret_cast<const uint4*>(kp + j * kstep + koff));
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) put(rg.v[j], *reinterpret_cast<const uint4*>(vp + voff[j]));
+            for (int j = 0; j < NJ; ++j) put(rg.v[j], *reinterpret_cast<const uint4*>(vp + j * vstep + voff));
         } else {
             issue(t, pi, rg);
         }
@@ -427,27 +421,116 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                 if (p.pack_lse) store_out(p.out, ob + D, lse_nat, p.out_dtype);
             }
         } else {
-            const int64_t row = ((int64_t)b * p.hq + hq) * p.num_splits + split;
+            const int64_t row = prow0 + (int64_t)g * prow_step;
             p.part_o[row * D + d] = res;
             if (d == 0) p.part_lse[row] = lse_nat;
         }
     }
 
-    };   // run_item
+    };   // run_piece
 
-    // ---- work distribution: one item per workgroup, or (persistent) a fixed set of workgroups that pull items
-    // from a queue: counters[0] is its head, counters[1] counts finished workgroups; the last one to finish
-    // puts both back to zero.  The first item of every workgroup is its own index.
-    int item = blockIdx.x;
-    while (item < p.total_items) {
-        run_item(item);
-        if (!p.persistent) return;
-        __syncthreads();
-        if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
-        __syncthreads();
-        item = s_next[0];
+    // ---- work distribution --------------------------------------------------------------------------------------
+    // Chunk mode: item -> (sequence, split, kv-head block, q-head tile), partial row (b, head, split); one item per
+    // workgroup, or (persistent) a fixed set of workgroups that pull items from a queue: counters[0] is its head,
+    // counters[1] counts finished workgroups, and the last one to finish puts both back to zero.  The first item
+    // of every workgroup is its own index.
+    // Balanced mode: the sequences, counted in granules of kGranule tokens and laid end to end, are cut into
+    // gridDim.x / units equal shares (fewer if there are fewer granules), units = (kv-head block, q-head tile)
+    // pairs of a sequence; workgroup (share wc, unit u) = blockIdx.x works its share off for its unit, sequence
+    // by sequence.  Its partial rows for sequence b go to slot (wc + b) * units + u: pieces are ordered by
+    // (wc, b) with at least one of the two growing from one piece to the next, so the slot is unique, and the
+    // pieces of a sequence occupy consecutive wc.  Neighbouring workgroups read the same tokens of neighbouring
+    // heads.  Every wavefront derives the same partition from kv_lens.
+    const int units = p.hg_blocks * p.head_tiles;
+    auto granules_of = [&](int bb) { return (max(min(p.kv_lens[bb], p.max_tokens), 0) + kGranule - 1) / kGranule; };
+    int item = blockIdx.x;                        // chunk mode: current item
+    int x = 0, hi = 0;                            // balanced mode: next granule, end of this workgroup's share
+    int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
+    const int wc = blockIdx.x / units, bu = blockIdx.x % units;
+    if (p.balanced) {
+        const int g_first = lane < p.batch ? granules_of(lane) : 0;          // sequences 0..63
+        const int incl_first = wave_scan_i32(g_first);
+        int total = __builtin_amdgcn_readlane(incl_first, 63);
+        for (int b0 = 64; b0 < p.batch; b0 += 64) total += wave_sum_i32(b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
+        const int shares = min((int)(gridDim.x / units), total);
+        if (wc >= shares) return;                                            // also total == 0
+        const int q = total / shares, r = total % shares;
+        x = wc * q + min(wc, r);
+        hi = x + q + (wc < r ? 1 : 0);
+        for (int b0 = 0, run = 0; b0 < p.batch; b0 += 64) {
+            const int g = b0 == 0 ? g_first : (b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
+            const int incl = b0 == 0 ? incl_first : wave_scan_i32(g);
+            const int excl = run + incl - g;
+            const uint64_t mask = __builtin_amdgcn_ballot_w64(g > 0 && excl <= x && x < excl + g);
+            if (mask) {
+                const int src = __builtin_ctzll(mask);
+                b = b0 + src;
+                before = __builtin_amdgcn_readlane(excl, src);
+                gb = __builtin_amdgcn_readlane(g, src);
+                break;
+            }
+            run += __builtin_amdgcn_readlane(incl, 63);
+        }
+    } else if (item >= p.total_items) {
+        return;
     }
-    if (threadIdx.x == 0) {
+    for (;;) {
+        int pb, hgb, ht, c_start, c_limit, prow_step;
+        int64_t prow0;
+        int piece_end = 0;
+        if (p.balanced) {
+            piece_end = min(before + gb, hi);
+            pb = b;
+            hgb = bu / p.head_tiles;
+            ht = bu % p.head_tiles;
+            c_start = (x - before) * kGranule;
+            c_limit = (piece_end - before) * kGranule;
+            const int64_t slot = (int64_t)(wc + b) * units + bu;
+            prow0 = slot * p.rows_per_slot + hl * p.heads_per_tile;
+            prow_step = 1;
+        } else {
+            int wg = item;
+            ht = wg % p.head_tiles;
+            wg /= p.head_tiles;
+            hgb = wg % p.hg_blocks;
+            wg /= p.hg_blocks;
+            const int split = wg % p.num_splits;
+            pb = wg / p.num_splits;
+            c_start = split * p.chunk;
+            c_limit = c_start + p.chunk;
+            prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
+            prow_step = p.num_splits;
+        }
+        // everything that describes the piece is wave-uniform: keep it in scalar registers
+        pb = __builtin_amdgcn_readfirstlane(pb);
+        hgb = __builtin_amdgcn_readfirstlane(hgb);
+        ht = __builtin_amdgcn_readfirstlane(ht);
+        c_start = __builtin_amdgcn_readfirstlane(c_start);
+        c_limit = __builtin_amdgcn_readfirstlane(c_limit);
+        prow_step = __builtin_amdgcn_readfirstlane(prow_step);
+        prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(prow0 >> 32)) << 32) |
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)prow0);
+        run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step);
+        if (p.balanced) {
+            x = piece_end;
+            if (x >= hi) return;
+            before += gb;                                             // on to the next sequence that has tokens
+            do {                                                      // one exists: granule x < hi is somewhere
+                b = min(b + 1, p.batch - 1);
+                gb = granules_of(b);
+            } while (gb == 0 && b + 1 < p.batch);
+            if (gb == 0) return;
+            __syncthreads();                                          // the LDS scratch is reused by the next piece
+        } else {
+            if (!p.persistent) return;
+            __syncthreads();
+            if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
+            __syncthreads();
+            item = s_next[0];
+            if (item >= p.total_items) break;
+        }
+    }
+    if (threadIdx.x == 0) {                       // persistent chunk mode: leave the counters at zero
         const int done = atomicAdd(p.counters + 1, 1);
         if (done == (int)gridDim.x - 1) {
             atomicExch(p.counters, 0);
@@ -475,8 +558,8 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // Persistent mode (work queue) whenever the KV range is split and the caller provided counters: items of a
     // ragged batch differ in length, and a queue keeps every compute unit busy until the end.
     const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
-    p.persistent = (p.counters != nullptr && !p.direct && p.total_items > resident) ? 1 : 0;
-    const dim3 grid((unsigned)(p.persistent ? resident : p.total_items));
+    p.persistent = (p.counters != nullptr && !p.direct && !p.balanced && p.total_items > resident) ? 1 : 0;
+    const dim3 grid((unsigned)(p.balanced ? p.workgroups : p.persistent ? resident : p.total_items));
     const dim3 block(64 * nw);
     // Two register buffers per wavefront, except for the widest rows where they would not leave room for two
     // workgroups per compute unit.

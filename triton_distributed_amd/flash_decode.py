@@ -72,10 +72,13 @@ def _stream_handle(stream) -> int:
 @dataclass
 class SplitKvPlan:
     """Shape-dependent launch constants (the role of the reference's ``algo_info`` dict)."""
-    num_splits: int
-    chunk_tokens: int
+    num_splits: int          # partial rows per (sequence, q head) the workspace holds; 1 = single pass
+    chunk_tokens: int        # tokens per split (chunk mode) / nominal tokens per workgroup (balanced mode)
     algo: str
     workspace_bytes: int
+    kv_heads_per_wg: int = 1
+    balanced: bool = False   # the kernel cuts the whole batch's KV ranges into equal shares from kv_lens
+    workgroups: int = 0
 
 
 def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -144,7 +147,8 @@ def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
     plan = FdkPlan()
     _lib.check(_LIB.fdk_plan(C.byref(a), num_cus, C.byref(plan)))
     ws = _LIB.fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits)
-    return SplitKvPlan(plan.num_splits, plan.chunk_tokens, _ALGO_NAMES[plan.algo], int(ws))
+    return SplitKvPlan(plan.num_splits, plan.chunk_tokens, _ALGO_NAMES[plan.algo], int(ws), plan.kv_heads_per_wg,
+                       bool(plan.balanced), plan.workgroups)
 
 
 def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, soft_cap=0.0, kv_split=-1,
@@ -249,7 +253,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         a.workspace = workspace.data_ptr()
         a.workspace_bytes = workspace.numel() * workspace.element_size()
-    if plan.num_splits > 1 and plan.algo == "mfma" and work_queue:
+    if plan.num_splits > 1 and plan.algo == "mfma" and work_queue and not plan.balanced:
         n_ctr = int(_LIB.fdk_counters_len(C.byref(a)))
         if counters is None:
             counters = torch.zeros(n_ctr, dtype=torch.int32, device=q.device)
