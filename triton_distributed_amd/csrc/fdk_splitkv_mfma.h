@@ -207,8 +207,15 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     // PM_TILE: a tile never leaves its page, so a load address is (page base + first slot of the tile), which
     // is wave-uniform, plus a per-lane byte offset that is the same for every full tile.
-    const uint32_t koff = (uint32_t)(((int64_t)lrow * p.k_st) * ES + lpiece * 16);   // per lane
-    const uint32_t voff = (uint32_t)(((int64_t)lrow * p.v_st) * ES + lpiece * 16);
+    // Per-lane byte offsets of the NJ loads.  Up to head_dim 128 they are kept in registers; the widest rows need
+    // the registers elsewhere and add a wave-uniform step per load instead (slightly slower).
+    constexpr bool kOffsetsInRegs = D <= 128;
+    uint32_t koff[kOffsetsInRegs ? NJ : 1], voff[kOffsetsInRegs ? NJ : 1];
+#pragma unroll
+    for (int j = 0; j < (kOffsetsInRegs ? NJ : 1); ++j) {
+        koff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.k_st) * ES + lpiece * 16);
+        voff[j] = (uint32_t)(((int64_t)(j * RPL + lrow) * p.v_st) * ES + lpiece * 16);
+    }
     const int64_t kstep = (int64_t)RPL * p.k_st * ES;                                 // per load, wave-uniform
     const int64_t vstep = (int64_t)RPL * p.v_st * ES;
     const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;   // wave-uniform
@@ -221,9 +228,11 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const char* kp = kplane + (pg * p.k_sp + (int64_t)slot0 * p.k_st) * ES;
             const char* vp = vplane + (pg * p.v_sp + (int64_t)slot0 * p.v_st) * ES;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) put(rg.k[j], *reinterpret_cast<const uint4*>(kp + j * kstep + koff));
+            for (int j = 0; j < NJ; ++j)
+                put(rg.k[j], *reinterpret_cast<const uint4*>(kOffsetsInRegs ? kp + koff[j] : kp + j * kstep + koff[0]));
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) put(rg.v[j], *reinterpret_cast<const uint4*>(vp + j * vstep + voff));
+            for (int j = 0; j < NJ; ++j)
+                put(rg.v[j], *reinterpret_cast<const uint4*>(kOffsetsInRegs ? vp + voff[j] : vp + j * vstep + voff[0]));
         } else {
             issue(t, pi, rg);
         }
@@ -441,6 +450,21 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     // (wc, b) with at least one of the two growing from one piece to the next, so the slot is unique, and the
     // pieces of a sequence occupy consecutive wc.  Neighbouring workgroups read the same tokens of neighbouring
     // heads.  Every wavefront derives the same partition from kv_lens.
+    if (!p.balanced && !p.persistent) {
+        // The common chunk-mode case is kept free of the loop below: straight-line code lets the compiler
+        // overlap the first loads of the piece (about a microsecond per workgroup on MI355X).
+        int wg = blockIdx.x;
+        if (wg >= p.total_items) return;
+        const int ht = wg % p.head_tiles;
+        wg /= p.head_tiles;
+        const int hgb = wg % p.hg_blocks;
+        wg /= p.hg_blocks;
+        const int split = wg % p.num_splits;
+        const int pb = wg / p.num_splits;
+        run_piece(pb, hgb, ht, split * p.chunk, split * p.chunk + p.chunk,
+                  ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split, p.num_splits);
+        return;
+    }
     const int units = p.hg_blocks * p.head_tiles;
     auto granules_of = [&](int bb) { return (max(min(p.kv_lens[bb], p.max_tokens), 0) + kGranule - 1) / kGranule; };
     int item = blockIdx.x;                        // chunk mode: current item
