@@ -204,6 +204,7 @@ def main():
             "workload": f"{args.config}: {inp.cfg.description}",
             "algorithmic_bytes_per_call": alg_bytes,
             "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
+            "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "kv_pools_rotated": len(pools),
         },
         "roofline": {
