@@ -43,6 +43,9 @@ def parse_args():
                     help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--op", default="decode", choices=["decode", "kv_append"],
+                    help="decode: the hot path (default); kv_append: the step before it (RMSNorm + rotary + "
+                         "paged append of one new token per sequence) at the same shape")
     return ap.parse_args()
 
 
@@ -99,6 +102,64 @@ def cpu_baseline(inp, budget_s: float):
     }
 
 
+def bench_kv_append(args):
+    """One new token per sequence of the configured shape through fdk_kv_append; latency-bound (a few KB per token)."""
+    import torch
+    import triton_distributed_amd as tda
+    from triton_distributed_amd import workloads as wl
+    cfg = wl.CONFIGS[args.config]
+    dev = torch.device("cuda:0")
+    b, hq, hkv, d, page = cfg.batch, cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.page_size
+    n = cfg.kv_len or cfg.kv_len_range[1]
+    g = torch.Generator().manual_seed(cfg.seed)
+    pages_per_seq = (n + page - 1) // page
+    pool = b * pages_per_seq
+    qkv = torch.randn(b, 1, hq + 2 * hkv, d, generator=g).to(torch.bfloat16).to(dev)
+    wq = (1.0 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16).to(dev)
+    wk = (1.0 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16).to(dev)
+    table = torch.randperm(pool, generator=g).to(torch.int32).view(b, pages_per_seq).to(dev)
+    lens = torch.full((b,), n, dtype=torch.int32, device=dev)
+    fp8 = cfg.kv_dtype == "fp8_e4m3"
+    kdt = torch.float8_e4m3fn if fp8 else torch.bfloat16
+    k = torch.zeros(pool, page, hkv, d, dtype=kdt, device=dev)
+    v = torch.zeros(pool, page, hkv, d, dtype=kdt, device=dev)
+    ks = torch.full((hkv,), 0.02, dtype=torch.float32, device=dev) if fp8 else None
+    freqs = torch.outer(torch.arange(n + 1, dtype=torch.float32),
+                        1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d)))
+    cos, sin = torch.cat((freqs, freqs), -1).cos().to(dev), torch.cat((freqs, freqs), -1).sin().to(dev)
+    q_out = torch.empty(b, 1, hq, d, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        tda.qk_norm_rope_update_kvcache(qkv, k, v, table, lens, wq, wk, cos, sin, q_out, k_scale=ks, v_scale=ks)
+
+    for _ in range(args.warmup):
+        step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
+    gpu_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    es = 1 if fp8 else 2
+    alg = b * (hq + 2 * hkv) * d * 2 + b * hq * d * 2 + 2 * b * hkv * d * es + 2 * b * (d // 2) * 4 + 2 * d * 2 + 8 * b
+    print(json.dumps({
+        "metric": f"kv-append (RMSNorm + rotary + paged write, 1 new token per sequence) us/call, {args.config} shape",
+        "value": round(wall_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if not fp8 else "bf16 -> fp8_e4m3 cache", "data": "synthetic (seeded N(0,1) bf16)",
+        "config": {"workload": f"{args.config}: B{b} {hq}q/{hkv}kv D{d} P{page}, position {n - 1}",
+                   "algorithmic_bytes_per_call": alg},
+        "roofline": {"bound": "hbm", "kernel": "kv_append_kernel", "achieved": round(alg / gpu_us / 1e3, 2),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(alg / gpu_us / 1e3 / HBM_PEAK_GBPS, 5),
+                     "us_per_launch": round(gpu_us, 2), "traffic": None,
+                     "note": "latency-bound: less than 1 MB per call"},
+    }), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -115,6 +176,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.op == "kv_append":
+        return bench_kv_append(args)
     t_gen = time.perf_counter()
     inp_cpu = wl.make_inputs(args.config)
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)

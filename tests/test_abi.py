@@ -12,7 +12,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "fdk.h")
 
 from triton_distributed_amd import _lib  # noqa: E402
-from triton_distributed_amd._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkPlan  # noqa: E402
+from triton_distributed_amd._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkPlan  # noqa: E402
 
 
 def _declared_functions():
@@ -43,7 +43,11 @@ int main(void) {
          offsetof(fdk_decode_args, counters_len));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
-  printf("%zu\n", sizeof(fdk_plan_t));
+  printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_kv_append_args), offsetof(fdk_kv_append_args, q_weight),
+         offsetof(fdk_kv_append_args, cos), offsetof(fdk_kv_append_args, max_positions),
+         offsetof(fdk_kv_append_args, block_table), offsetof(fdk_kv_append_args, k_cache),
+         offsetof(fdk_kv_append_args, k_scale), offsetof(fdk_kv_append_args, q_out_stride_h));
   return 0;
 }''')
     exe = tmp_path / "layout"
@@ -59,7 +63,12 @@ int main(void) {
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
                                              ("partial_lse", "kv_lens", "lse_stride_b_out")]
     assert got == want
-    assert int(lines[2]) == C.sizeof(FdkPlan)
+    assert [int(x) for x in lines[2].split()] == [C.sizeof(FdkPlan), FdkPlan.balanced.offset, FdkPlan.workgroups.offset]
+    got = [int(x) for x in lines[3].split()]
+    want = [C.sizeof(FdkKvAppendArgs)] + [getattr(FdkKvAppendArgs, f).offset for f in
+                                         ("q_weight", "cos", "max_positions", "block_table", "k_cache", "k_scale",
+                                          "q_out_stride_h")]
+    assert got == want
 
 
 def _args(**kw):
@@ -247,3 +256,61 @@ def test_combine_ranks_validation():
     a.num_ranks = 0
     assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
     assert lib.fdk_combine_ranks(None, None) == _lib.FDK_ENULL
+
+
+def _append_args(**kw):
+    """A valid dry-run fdk_kv_append block on fake pointers: B32, 1 new token, 32q/8kv, D128, P16."""
+    a = FdkKvAppendArgs()
+    a.struct_size = C.sizeof(FdkKvAppendArgs)
+    a.flags = _lib.FDK_FLAG_DRY_RUN
+    a.qkv, a.q_weight, a.k_weight, a.cos, a.sin = 0x10000, 0x20000, 0x30000, 0x40000, 0x50000
+    a.qkv_stride_b, a.qkv_stride_t, a.qkv_stride_h = 48 * 128, 48 * 128, 128
+    a.qkv_dtype = a.kv_dtype = _lib.FDK_BF16
+    a.q_eps = a.k_eps = 1e-6
+    a.cs_stride_b, a.cs_stride_pos, a.max_positions = 0, 128, 8192
+    a.batch, a.new_tokens, a.num_q_heads, a.num_kv_heads, a.head_dim = 32, 1, 32, 8, 128
+    a.block_table, a.table_stride_b, a.kv_lens = 0x60000, 256, 0x70000
+    a.page_size, a.max_pages, a.num_pages = 16, 256, 9000
+    a.k_cache, a.v_cache = 0x80000, 0x90000
+    a.k_stride_page = a.v_stride_page = 16 * 8 * 128
+    a.k_stride_tok = a.v_stride_tok = 8 * 128
+    a.k_stride_head = a.v_stride_head = 128
+    a.q_out, a.q_out_stride_b, a.q_out_stride_t, a.q_out_stride_h = 0xA0000, 32 * 128, 32 * 128, 128
+    for k, v in kw.items():
+        setattr(a, k, v)
+    return a
+
+
+def test_kv_append_accepts_valid_arguments_and_rejects_bad_ones():
+    lib = _lib.load()
+    assert lib.fdk_kv_append(C.byref(_append_args()), None) == 0, lib.fdk_last_error()
+    assert lib.fdk_kv_append(C.byref(_append_args(kv_dtype=_lib.FDK_FP8_E4M3, k_scale=0xB0000, v_scale=0xC0000)), None) == 0
+    assert lib.fdk_kv_append(C.byref(_append_args(batch=0, qkv=None)), None) == 0         # nothing to do
+    assert lib.fdk_kv_append(None, None) == _lib.FDK_ENULL
+    for field, value, code in [
+        ("struct_size", 8, _lib.FDK_EABI),
+        ("head_dim", 96, _lib.FDK_EUNSUPPORTED),
+        ("qkv_dtype", _lib.FDK_FP32, _lib.FDK_EUNSUPPORTED),
+        ("kv_dtype", _lib.FDK_FP16, _lib.FDK_EUNSUPPORTED),
+        ("kv_dtype", _lib.FDK_FP8_E4M3, _lib.FDK_ENULL),              # fp8 cache without scales
+        ("qkv", None, _lib.FDK_ENULL),
+        ("cos", None, _lib.FDK_ENULL),
+        ("q_out", None, _lib.FDK_ENULL),
+        ("k_cache", None, _lib.FDK_ENULL),
+        ("num_kv_heads", 0, _lib.FDK_ESHAPE),
+        ("new_tokens", -1, _lib.FDK_ESHAPE),
+        ("page_size", 0, _lib.FDK_ESHAPE),
+        ("num_pages", 0, _lib.FDK_ESHAPE),
+        ("max_positions", 0, _lib.FDK_ESHAPE),
+        ("qkv_stride_h", 64, _lib.FDK_ESHAPE),
+        ("q_out_stride_h", 127, _lib.FDK_ESHAPE),
+        ("cs_stride_pos", 32, _lib.FDK_ESHAPE),
+        ("table_stride_b", 255, _lib.FDK_ESHAPE),
+        ("k_stride_head", 64, _lib.FDK_ESHAPE),
+        ("v_stride_tok", -8, _lib.FDK_ESHAPE),
+        ("q_eps", float("nan"), _lib.FDK_ESHAPE),
+        ("k_eps", -1.0, _lib.FDK_ESHAPE),
+    ]:
+        rc = lib.fdk_kv_append(C.byref(_append_args(**{field: value})), None)
+        assert rc == code, (field, value, rc, lib.fdk_last_error())
+        assert lib.fdk_last_error() != b""

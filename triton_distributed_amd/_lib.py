@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 3
+FDK_ABI_VERSION = 4
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -24,7 +24,7 @@ FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN = 1, 2
 
 EXPORTS = (
     "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
-    "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len",
+    "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len", "fdk_kv_append",
 )
 
 
@@ -64,6 +64,27 @@ class FdkCombineRanksArgs(C.Structure):
         ("num_ranks", C.c_int32), ("batch", C.c_int32), ("num_q_heads", C.c_int32), ("head_dim", C.c_int32),
         ("out", C.c_void_p), ("out_stride_b", C.c_int64), ("out_stride_h", C.c_int64),
         ("lse", C.c_void_p), ("lse_stride_b_out", C.c_int64),
+    ]
+
+
+class FdkKvAppendArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("flags", C.c_uint32),
+        ("qkv", C.c_void_p), ("qkv_stride_b", C.c_int64), ("qkv_stride_t", C.c_int64), ("qkv_stride_h", C.c_int64),
+        ("qkv_dtype", C.c_int32), ("kv_dtype", C.c_int32),
+        ("q_weight", C.c_void_p), ("k_weight", C.c_void_p), ("q_eps", C.c_float), ("k_eps", C.c_float),
+        ("cos", C.c_void_p), ("sin", C.c_void_p), ("cs_stride_b", C.c_int64), ("cs_stride_pos", C.c_int64),
+        ("max_positions", C.c_int32),
+        ("batch", C.c_int32), ("new_tokens", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("block_table", C.c_void_p), ("table_stride_b", C.c_int64), ("kv_lens", C.c_void_p),
+        ("page_size", C.c_int32), ("max_pages", C.c_int32), ("num_pages", C.c_int32),
+        ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("k_stride_page", C.c_int64), ("k_stride_tok", C.c_int64), ("k_stride_head", C.c_int64),
+        ("v_stride_page", C.c_int64), ("v_stride_tok", C.c_int64), ("v_stride_head", C.c_int64),
+        ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+        ("q_out", C.c_void_p), ("q_out_stride_b", C.c_int64), ("q_out_stride_t", C.c_int64),
+        ("q_out_stride_h", C.c_int64),
     ]
 
 
@@ -109,6 +130,8 @@ def load() -> C.CDLL:
     lib.fdk_counters_len.argtypes = [C.POINTER(FdkDecodeArgs)]
     lib.fdk_combine_ranks.restype = C.c_int
     lib.fdk_combine_ranks.argtypes = [C.POINTER(FdkCombineRanksArgs), C.c_void_p]
+    lib.fdk_kv_append.restype = C.c_int
+    lib.fdk_kv_append.argtypes = [C.POINTER(FdkKvAppendArgs), C.c_void_p]
     if lib.fdk_abi_version() != FDK_ABI_VERSION:
         raise ImportError(f"{path}: ABI version {lib.fdk_abi_version()} != {FDK_ABI_VERSION}")
     _lib = lib

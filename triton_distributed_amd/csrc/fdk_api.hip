@@ -433,4 +433,64 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
     return FDK_OK;
 }
 
+int fdk_kv_append(const fdk_kv_append_args* a, void* hip_stream) {
+    g_err[0] = 0;
+    if (!a) return fail(FDK_ENULL, "args is null");
+    if (a->struct_size != sizeof(fdk_kv_append_args))
+        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_kv_append_args));
+    if (a->batch < 0 || a->new_tokens < 0) return fail(FDK_ESHAPE, "batch %d / new_tokens %d < 0", a->batch, a->new_tokens);
+    if (a->num_q_heads < 0 || a->num_kv_heads <= 0)
+        return fail(FDK_ESHAPE, "bad head counts Hq=%d Hkv=%d", a->num_q_heads, a->num_kv_heads);
+    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
+        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
+    if (a->qkv_dtype != FDK_BF16 && a->qkv_dtype != FDK_FP16)
+        return fail(FDK_EUNSUPPORTED, "qkv_dtype %d (bf16 or fp16 only)", a->qkv_dtype);
+    if (a->kv_dtype != a->qkv_dtype && a->kv_dtype != FDK_FP8_E4M3)
+        return fail(FDK_EUNSUPPORTED, "kv_dtype %d must equal qkv_dtype or be fp8_e4m3", a->kv_dtype);
+    if (a->page_size <= 0 || a->max_pages <= 0 || a->num_pages <= 0)
+        return fail(FDK_ESHAPE, "page_size %d, max_pages %d, num_pages %d must be positive", a->page_size, a->max_pages,
+                    a->num_pages);
+    if ((int64_t)a->max_pages * a->page_size > INT32_MAX) return fail(FDK_ESHAPE, "max_pages*page_size overflows int32");
+    if (a->max_positions <= 0) return fail(FDK_ESHAPE, "max_positions %d <= 0", a->max_positions);
+    if (!(a->q_eps == a->q_eps) || !(a->k_eps == a->k_eps) || a->q_eps < 0.f || a->k_eps < 0.f)
+        return fail(FDK_ESHAPE, "eps must be non-negative numbers");
+    if (a->batch == 0 || a->new_tokens == 0) return FDK_OK;
+    if ((int64_t)a->batch * a->new_tokens * (a->num_q_heads + 2 * a->num_kv_heads) > (int64_t)INT32_MAX * 4)
+        return fail(FDK_ESHAPE, "grid too large");
+    if (!a->qkv || !a->k_weight || !a->cos || !a->sin || !a->block_table || !a->kv_lens || !a->k_cache || !a->v_cache)
+        return fail(FDK_ENULL, "qkv / k_weight / cos / sin / block_table / kv_lens / k_cache / v_cache must be non-null");
+    if (a->num_q_heads > 0 && (!a->q_weight || !a->q_out)) return fail(FDK_ENULL, "q_weight / q_out is null");
+    if (a->kv_dtype == FDK_FP8_E4M3 && (!a->k_scale || !a->v_scale))
+        return fail(FDK_ENULL, "k_scale / v_scale are required for an fp8 cache");
+    if (a->qkv_stride_h < a->head_dim) return fail(FDK_ESHAPE, "qkv_stride_h %lld < head_dim", (long long)a->qkv_stride_h);
+    if (a->num_q_heads > 0 && a->q_out_stride_h < a->head_dim)
+        return fail(FDK_ESHAPE, "q_out_stride_h %lld < head_dim", (long long)a->q_out_stride_h);
+    if (a->cs_stride_pos < a->head_dim / 2) return fail(FDK_ESHAPE, "cos/sin rows shorter than head_dim/2");
+    if (a->table_stride_b < a->max_pages)
+        return fail(FDK_ESHAPE, "table_stride_b %lld < max_pages %d", (long long)a->table_stride_b, a->max_pages);
+    const int64_t st[6] = {a->k_stride_page, a->k_stride_tok, a->k_stride_head,
+                           a->v_stride_page, a->v_stride_tok, a->v_stride_head};
+    for (int i = 0; i < 6; ++i)
+        if (st[i] < 0) return fail(FDK_ESHAPE, "negative cache stride");
+    if (a->num_kv_heads > 1 && (a->k_stride_head < a->head_dim || a->v_stride_head < a->head_dim))
+        return fail(FDK_ESHAPE, "cache head stride < head_dim");
+    if (a->flags & FDK_FLAG_DRY_RUN) return FDK_OK;
+    fdk::KvAppendParams p;
+    memset(&p, 0, sizeof(p));
+    p.qkv = a->qkv; p.q_weight = a->q_weight; p.k_weight = a->k_weight; p.cos = a->cos; p.sin = a->sin;
+    p.block_table = a->block_table; p.kv_lens = a->kv_lens; p.k_scale = a->k_scale; p.v_scale = a->v_scale;
+    p.k_cache = a->k_cache; p.v_cache = a->v_cache; p.q_out = a->q_out;
+    p.qkv_sb = a->qkv_stride_b; p.qkv_st = a->qkv_stride_t; p.qkv_sh = a->qkv_stride_h;
+    p.cs_sb = a->cs_stride_b; p.cs_sp = a->cs_stride_pos; p.tbl_sb = a->table_stride_b;
+    p.k_sp = a->k_stride_page; p.k_st = a->k_stride_tok; p.k_sh = a->k_stride_head;
+    p.v_sp = a->v_stride_page; p.v_st = a->v_stride_tok; p.v_sh = a->v_stride_head;
+    p.qo_sb = a->q_out_stride_b; p.qo_st = a->q_out_stride_t; p.qo_sh = a->q_out_stride_h;
+    p.batch = a->batch; p.new_tokens = a->new_tokens; p.hq = a->num_q_heads; p.hkv = a->num_kv_heads;
+    p.head_dim = a->head_dim; p.page_size = a->page_size; p.max_pages = a->max_pages; p.num_pages = a->num_pages;
+    p.max_positions = a->max_positions; p.q_eps = a->q_eps; p.k_eps = a->k_eps;
+    int rc = fdk::launch_kv_append(p, a->qkv_dtype, a->kv_dtype, reinterpret_cast<hipStream_t>(hip_stream));
+    if (rc) return fail(rc, "kv append launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
 }  // extern "C"

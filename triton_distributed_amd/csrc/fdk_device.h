@@ -81,7 +81,31 @@ struct CombineRanksParams {
     int32_t partial_dtype, out_dtype, packed;
 };
 
+struct KvAppendParams {
+    const void* qkv;
+    const void* q_weight;
+    const void* k_weight;
+    const float* cos;
+    const float* sin;
+    const int32_t* block_table;
+    const int32_t* kv_lens;
+    const float* k_scale;
+    const float* v_scale;
+    void* k_cache;
+    void* v_cache;
+    void* q_out;
+    int64_t qkv_sb, qkv_st, qkv_sh;
+    int64_t cs_sb, cs_sp;
+    int64_t tbl_sb;
+    int64_t k_sp, k_st, k_sh, v_sp, v_st, v_sh;
+    int64_t qo_sb, qo_st, qo_sh;
+    int32_t batch, new_tokens, hq, hkv, head_dim;
+    int32_t page_size, max_pages, num_pages, max_positions;
+    float q_eps, k_eps;
+};
+
 // Launchers implemented in the .hip files; return hipError_t as int.
+int launch_kv_append(const KvAppendParams& p, int qkv_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_combine(const CombineParams& p, hipStream_t stream);

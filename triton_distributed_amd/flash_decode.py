@@ -39,7 +39,7 @@ from typing import Optional, Sequence, Tuple, Union
 import torch
 
 from . import _lib
-from ._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkPlan
+from ._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkPlan
 
 _LIB = _lib.load()          # raises ImportError when libfdk.so is not built - by design
 
@@ -403,3 +403,84 @@ def inter_rank_combine(all_ranks_output: torch.Tensor, global_kv_lens: torch.Ten
         a.lse_stride_b_out = lse_out.stride(0)
     _lib.check(_LIB.fdk_combine_ranks(C.byref(a), _stream_handle(stream)))
     return final_output
+
+
+def qk_norm_rope_update_kvcache(qkv: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                                block_tables: torch.Tensor, kv_lens: torch.Tensor, q_rms_weight: torch.Tensor,
+                                k_rms_weight: torch.Tensor, cos_cache: torch.Tensor, sin_cache: torch.Tensor,
+                                q_norm_rope: Optional[torch.Tensor] = None, q_rms_eps: float = 1e-6,
+                                k_rms_eps: float = 1e-6, *, k_scale: Optional[torch.Tensor] = None,
+                                v_scale: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """The step before the decode: per-head RMSNorm and rotary embedding of the new tokens' q and k rows, and the
+    append of their K / V rows to the paged cache.  Argument order of the reference's
+    ``ModelBuilder.make_qk_norm_rope_update_kvcache`` (mega_triton_kernel/models/model_builder.py:341-345).
+
+    qkv          [B, T, Hq + 2 Hkv, D] bf16/fp16: q heads, k heads, v heads of the T new tokens
+    key_cache    [num_pages, P, Hkv, D] in qkv's dtype or float8_e4m3fn (then with k_scale / v_scale [Hkv] fp32);
+    value_cache  updated in place at positions ``kv_lens[b] - T + t``
+    block_tables [B, max_pages] int32;  kv_lens [B] int32, ALREADY counting the new tokens (model_builder.py:347)
+    q/k_rms_weight [D] in qkv's dtype;  cos_cache / sin_cache [S, D], [1, S, D] or [B, S, D] fp32, row = position
+    Returns ``q_norm_rope [B, T, Hq, D]`` - the query the decode takes (reshape to [B, Hq, D] for T = 1)."""
+    if qkv.dim() != 4 or key_cache.dim() != 4 or value_cache.dim() != 4:
+        raise ValueError("qkv must be [B, T, heads, D]; caches [num_pages, P, Hkv, D]")
+    batch, new_tokens, heads, d = qkv.shape
+    num_pages, page_size, kv_heads, dk = key_cache.shape
+    if dk != d or tuple(value_cache.shape) != tuple(key_cache.shape) or key_cache.dtype != value_cache.dtype:
+        raise ValueError("caches must share shape and dtype, with qkv's head_dim")
+    q_heads = heads - 2 * kv_heads
+    if q_heads < 0:
+        raise ValueError(f"qkv has {heads} heads, fewer than 2 * {kv_heads} kv heads")
+    fp8 = key_cache.dtype == torch.float8_e4m3fn
+    if not fp8 and key_cache.dtype != qkv.dtype:
+        raise ValueError("a 16-bit cache must have qkv's dtype")
+    if fp8 and (k_scale is None or v_scale is None):
+        raise ValueError("k_scale / v_scale are required for an fp8 cache")
+    for name, tns in (("qkv", qkv), ("key_cache", key_cache), ("value_cache", value_cache)):
+        if tns.stride(-1) != 1:
+            raise ValueError(f"{name}: the head dimension must be contiguous")
+        if not tns.is_cuda:
+            raise ValueError(f"{name} must live on the GPU; there is no CPU path")
+    for name, w in (("q_rms_weight", q_rms_weight), ("k_rms_weight", k_rms_weight)):
+        if w.dtype != qkv.dtype or tuple(w.shape) != (d,) or not w.is_contiguous() or not w.is_cuda:
+            raise ValueError(f"{name} must be a contiguous [{d}] GPU tensor of qkv's dtype")
+    if cos_cache.shape != sin_cache.shape or cos_cache.dtype != torch.float32 or sin_cache.dtype != torch.float32 or \
+            cos_cache.stride() != sin_cache.stride() or not cos_cache.is_cuda or not sin_cache.is_cuda:
+        raise ValueError("cos_cache and sin_cache must be fp32 GPU tensors of one shape and layout")
+    cs = cos_cache if cos_cache.dim() == 3 else cos_cache[None]
+    if cs.dim() != 3 or cs.shape[0] not in (1, batch) or cs.shape[-1] < d // 2 or cs.stride(-1) != 1:
+        raise ValueError("cos_cache / sin_cache must be [S, D], [1, S, D] or [B, S, D]")
+    if block_tables.dtype != torch.int32 or kv_lens.dtype != torch.int32 or block_tables.dim() != 2 or \
+            block_tables.shape[0] != batch or block_tables.stride(-1) != 1 or tuple(kv_lens.shape) != (batch,) or \
+            not kv_lens.is_contiguous() or not block_tables.is_cuda or not kv_lens.is_cuda:
+        raise ValueError("block_tables [B, max_pages] and kv_lens [B] must be contiguous int32 GPU tensors")
+    if q_norm_rope is None:
+        q_norm_rope = torch.empty((batch, new_tokens, q_heads, d), dtype=qkv.dtype, device=qkv.device)
+    elif tuple(q_norm_rope.shape) != (batch, new_tokens, q_heads, d) or q_norm_rope.dtype != qkv.dtype or \
+            q_norm_rope.stride(-1) != 1 or not q_norm_rope.is_cuda:
+        raise ValueError(f"q_norm_rope must be a GPU tensor [{batch}, {new_tokens}, {q_heads}, {d}] of qkv's dtype")
+    a = FdkKvAppendArgs()
+    a.struct_size = C.sizeof(FdkKvAppendArgs)
+    a.qkv = qkv.data_ptr()
+    a.qkv_stride_b, a.qkv_stride_t, a.qkv_stride_h = qkv.stride(0), qkv.stride(1), qkv.stride(2)
+    a.qkv_dtype = _fdk_dtype(qkv.dtype, "qkv")
+    a.kv_dtype = _fdk_dtype(key_cache.dtype, "key_cache")
+    a.q_weight, a.k_weight = q_rms_weight.data_ptr(), k_rms_weight.data_ptr()
+    a.q_eps, a.k_eps = float(q_rms_eps), float(k_rms_eps)
+    a.cos, a.sin = cos_cache.data_ptr(), sin_cache.data_ptr()
+    a.cs_stride_b = cs.stride(0) if cs.shape[0] > 1 else 0
+    a.cs_stride_pos, a.max_positions = cs.stride(1), cs.shape[1]
+    a.batch, a.new_tokens, a.num_q_heads, a.num_kv_heads, a.head_dim = batch, new_tokens, q_heads, kv_heads, d
+    a.block_table, a.table_stride_b, a.kv_lens = block_tables.data_ptr(), block_tables.stride(0), kv_lens.data_ptr()
+    a.page_size, a.max_pages, a.num_pages = page_size, block_tables.shape[1], num_pages
+    a.k_cache, a.v_cache = key_cache.data_ptr(), value_cache.data_ptr()
+    a.k_stride_page, a.k_stride_tok, a.k_stride_head = key_cache.stride(0), key_cache.stride(1), key_cache.stride(2)
+    a.v_stride_page, a.v_stride_tok, a.v_stride_head = value_cache.stride(0), value_cache.stride(1), value_cache.stride(2)
+    if fp8:
+        for name, sc in (("k_scale", k_scale), ("v_scale", v_scale)):
+            if sc.dtype != torch.float32 or tuple(sc.shape) != (kv_heads,) or not sc.is_contiguous() or not sc.is_cuda:
+                raise ValueError(f"{name} must be a contiguous fp32 GPU tensor [{kv_heads}]")
+        a.k_scale, a.v_scale = k_scale.data_ptr(), v_scale.data_ptr()
+    a.q_out = q_norm_rope.data_ptr()
+    a.q_out_stride_b, a.q_out_stride_t, a.q_out_stride_h = q_norm_rope.stride(0), q_norm_rope.stride(1), q_norm_rope.stride(2)
+    _lib.check(_LIB.fdk_kv_append(C.byref(a), _stream_handle(stream)))
+    return q_norm_rope
