@@ -15,6 +15,8 @@ closed_form     float64 brute force of ``(out, lse)``, the split/combine
                 textbook log-sum-exp merge they must reduce to.
 fp8             OCP e4m3fn decode table and the per-kv-head dequantisation the
                 fp8 KV-cache workload is defined by.
+kv_append       the step before the path: per-head RMSNorm, rotary embedding and
+                the paged KV-cache append (restates the reference's Triton kernel).
 
 Pinning status (what checks the oracle itself; see tests/test_oracle_*.py):
   * paged_attn.ref_paged_attn      pinned: agrees with closed_form.attn_fp64 within the
@@ -30,4 +32,9 @@ Pinning status (what checks the oracle itself; see tests/test_oracle_*.py):
                                    logsumexp/softmax identity, -inf (empty) entries.
   * fp8.e4m3fn_table               pinned: exhaustive 256-entry comparison with
                                    torch.float8_e4m3fn CPU casts and the OCP bit formula.
+  * kv_append.kv_append            pinned at the reference test's 1e-2 tolerance against an independent
+                                   float64 route (numpy norm, complex rotation), rotation invariants,
+                                   bit-exact copies / untouched rows; the bf16 rounding points of the
+                                   reference's Triton kernel beyond that tolerance are "parity unpinned"
+                                   (its own oracle, flashinfer, is not available and it stores no vectors).
 """
