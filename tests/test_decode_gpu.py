@@ -374,6 +374,56 @@ def test_runs_on_a_side_stream_and_is_repeatable(cuda_device):
     assert torch.equal(o0, o1) and torch.equal(l0, l1)      # deterministic: no atomics, fixed merge order
 
 
+@pytest.mark.parametrize("mode", ["single_pass", "chunks_queue", "balanced"])
+def test_hip_graph_replays_follow_the_inputs(cuda_device, mode):
+    # A captured call holds only pointers: replays must follow in-place changes of q and kv_lens (also the
+    # balanced partition, which the kernel derives from kv_lens), with eager work between the replays.
+    g = torch.Generator().manual_seed(61)
+    if mode == "single_pass":
+        b, hq, hkv, n_max, kw = 40, 32, 8, 700, {}
+    elif mode == "chunks_queue":
+        b, hq, hkv, n_max, kw = 12, 32, 8, 3000, dict(kv_split=24)        # 12*24*4 items > 512 resident workgroups
+    else:
+        b, hq, hkv, n_max, kw = 3, 8, 1, 40000, {}
+    d, page = 128, 16
+    pages = (n_max + page - 1) // page
+    pool = b * pages
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.randperm(pool, generator=g).to(torch.int32).view(b, pages).to(cuda_device)
+    lens_sets = [torch.randint(1, n_max + 1, (b,), generator=g).to(torch.int32) for _ in range(3)]
+    lens_sets[1][0] = 0                                                        # an empty sequence in one replay
+    lens_t = lens_sets[0].clone().to(cuda_device)
+    call = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=n_max, **kw)
+    if mode == "balanced":
+        assert call.plan.balanced
+    elif mode == "single_pass":
+        assert call.plan.num_splits == 1
+    else:
+        assert call.plan.num_splits == 24 and not call.plan.balanced
+    call.run()                                                                  # warm up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call.run()
+    for i, new_lens in enumerate(lens_sets):
+        lens_t.copy_(new_lens.to(cuda_device))
+        q.copy_(torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device))
+        call.out.fill_(float("nan"))
+        call.lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_o, got_l = call.out.clone(), call.lse.clone()
+        want_o, want_l = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=n_max, **kw)   # eager, own buffers
+        torch.cuda.synchronize()
+        assert torch.equal(got_o, want_o) and torch.equal(got_l, want_l), f"replay {i}"
+        live = [j for j in range(b) if int(new_lens[j]) > 0]
+        rows = live[:4]
+        _check(got_o[rows], got_l[rows], q[rows], k, v, table[rows], [int(new_lens[j]) for j in rows], d ** -0.5,
+               tag=f"graph replay {i}")
+
+
 def test_inter_rank_combine_equals_one_shot(cuda_device):
     # R ranks each hold a disjoint slice of every sequence (sequence parallel decode, one GPU stands in for all):
     # local decode per rank -> packed [R,B,Hq,D+1] -> merge == decode over the whole sequence
