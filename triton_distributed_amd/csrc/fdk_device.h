@@ -193,6 +193,12 @@ template <> struct Pack2<FDK_BF16> {
         vec r = {(__bf16)a, (__bf16)b};
         return __builtin_bit_cast(uint32_t, r);
     }
+    // bytes 0,1 (hi = false) or 2,3 (hi = true) of four e4m3 values, converted exactly, in one instruction
+    // (v_cvt_scalef32_pk_bf16_fp8 applies only the exponent of its scale operand; 1.0 leaves the value alone)
+    static __device__ __forceinline__ uint32_t from_fp8(uint32_t four, bool hi) {
+        return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, 1.0f, true)
+                                               : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, 1.0f, false));
+    }
 };
 template <> struct Pack2<FDK_FP16> {
     using vec = f16x2_t;
@@ -204,6 +210,10 @@ template <> struct Pack2<FDK_FP16> {
     static __device__ __forceinline__ uint32_t pack(float a, float b) {
         vec r = {(_Float16)a, (_Float16)b};
         return __builtin_bit_cast(uint32_t, r);
+    }
+    static __device__ __forceinline__ uint32_t from_fp8(uint32_t four, bool hi) {
+        return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, 1.0f, true)
+                                               : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, 1.0f, false));
     }
 };
 

@@ -258,10 +258,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                     ko[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
                     ko[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
                     // V: exact conversion; its scale multiplies the output once at the end
-                    const f32x2_t v01 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.v[j][w], false);
-                    const f32x2_t v23 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.v[j][w], true);
-                    vo[2 * w] = P2::pack(v01.x, v01.y);
-                    vo[2 * w + 1] = P2::pack(v23.x, v23.y);
+                    vo[2 * w] = P2::from_fp8(rg.v[j][w], false);
+                    vo[2 * w + 1] = P2::from_fp8(rg.v[j][w], true);
                 }
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {

@@ -290,10 +290,13 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
     and lse = ln sum exp(scaled logits) - what the cross-rank combine consumes."""
+    if q.is_cuda:
+        stream = _stream_handle(stream)               # looked up once: torch.cuda.current_stream() is not free
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
                           out=out, lse=lse, workspace=workspace, algo=algo,
-                          counters=_stream_counters(q.device, stream))
+                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
+                          work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)
 
 
@@ -307,9 +310,12 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
     batch, q_heads, d = q.shape
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
+    if q.is_cuda:
+        stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
-                          want_lse=False, counters=_stream_counters(q.device, stream))
+                          want_lse=False, counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
+                          work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     call.run(stream)
     return output_combine
 
@@ -317,9 +323,12 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
 def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
                          output_split=None, output_combine=None, kv_split=-1, stream=None):
     """Drop-in for the reference function of the same name (flash_decode.py:763-844): ``[B, Hq, D]``."""
+    if q.is_cuda:
+        stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
-                          want_lse=False, counters=_stream_counters(q.device, stream))
+                          want_lse=False, counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
+                          work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)[0]
 
 
