@@ -87,6 +87,32 @@ def test_reference_grid(cuda_device, kv_lens, num_heads, block_size, dtype, soft
     torch.testing.assert_close(packed[..., d].float(), lse, atol=3e-2, rtol=1e-2)     # lse rounded to 16 bits
 
 
+# ---- the reference's persistent entry point and its test grid (test_decode_attn.py:207-251, 254-296) --------------
+@pytest.mark.parametrize("kv_lens", [[32], [1320], [18], [463], [1], [54], [293], [70], [1320, 18, 463, 1, 4000] * 8])
+def test_persistent_entry_points(cuda_device, kv_lens):
+    hq, hkv, d, block_size, dtype = 96, 12, 128, 1, torch.float16
+    num_blocks = 8192
+    g = torch.Generator().manual_seed(len(kv_lens) * 1000 + kv_lens[0])
+    q = torch.randn(len(kv_lens), hq, d, generator=g).to(dtype).to(cuda_device)
+    kv = torch.randn(num_blocks, 2, block_size, hkv, d, generator=g).to(dtype).to(cuda_device)
+    k, v = kv[:, 0].contiguous(), kv[:, 1].contiguous()
+    table = torch.randint(0, num_blocks, (len(kv_lens), max(kv_lens)), generator=g, dtype=torch.int32).to(cuda_device)
+    lens_t = _lens_t(kv_lens, cuda_device)
+    scale = d ** -0.5
+    ws1 = torch.zeros([1], dtype=torch.int32, device=cuda_device)       # what the reference's test passes
+    ws4 = torch.zeros([4], dtype=torch.int32, device=cuda_device)       # large enough to serve as the queue counters
+    out = tda.gqa_fwd_batch_decode_persistent(q, k, v, ws1, [1] * len(kv_lens), lens_t, table, scale, 0)
+    out4 = tda.gqa_fwd_batch_decode_persistent(q, k, v, ws4, [1] * len(kv_lens), lens_t, table, scale, 0)
+    out_aot = tda.gqa_fwd_batch_decode_persistent_aot(torch.cuda.current_stream(), q, k, v, ws1, [1] * len(kv_lens),
+                                                      lens_t, table, scale, 0, kv_split=16)
+    torch.cuda.synchronize()
+    assert out.shape == (len(kv_lens), hq, d) and out.dtype == dtype
+    ref = ref_paged_attn(q, k, v, kv_lens, table, scale, 0.0)
+    for o in (out, out4, out_aot):
+        torch.testing.assert_close(o.float(), ref.float(), atol=1e-2, rtol=1e-2)        # the reference test's bar
+    assert torch.equal(out, out4) and int(ws4.abs().sum()) == 0 and int(ws1.abs().sum()) == 0
+
+
 def test_large_pool_index_arithmetic(cuda_device):
     # NUM_BLOCKS = 32000 "large enough to test overflow in index calculation" (test_decode_attn.py:120):
     # here the pool is made large enough that element offsets pass 2^31 and 2^32

@@ -346,6 +346,33 @@ def gqa_fwd_batch_decode_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_
                                 output_split, output_combine, kv_split, stream=stream)
 
 
+def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0,
+                                    output_split=None, output_combine=None, kv_split=-1, stream=None):
+    """Drop-in for the reference function of the same name (flash_decode.py:931-976): ``[B, Hq, D]``.
+
+    The reference runs a fixed grid of 132 programs that loop over (sequence, head, split) items and merge after a
+    grid barrier on the int32 ``workspace``.  Here the same split count (32 unless ``kv_split`` says otherwise) runs
+    as the work-queue form of the split kernel - two workgroups per compute unit pulling items - followed by the
+    combine kernel.  ``workspace`` is used as the queue's counters when it is a zeroed int32 GPU tensor with at
+    least two elements (the kernel leaves it zero); otherwise per-stream counters of this module are used.  The
+    result is in q's dtype (the reference allocates float16 whatever q is)."""
+    splits = 32 if kv_split == -1 else kv_split
+    if q.is_cuda:
+        stream = _stream_handle(stream)
+    ctr = workspace if (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.dtype == torch.int32 and
+                        workspace.numel() >= 2 and workspace.is_contiguous()) else _stream_counters(q.device, stream)
+    call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap, kv_split=splits,
+                          workspace=_as_scratch(output_split), out=output_combine, want_lse=False, counters=ctr)
+    return call.run(stream)[0]
+
+
+def gqa_fwd_batch_decode_persistent_aot(stream, q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
+                                        soft_cap=0, output_split=None, output_combine=None, kv_split=-1):
+    """Stream-first form (flash_decode.py:1095-1150)."""
+    return gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap,
+                                           output_split, output_combine, kv_split, stream=stream)
+
+
 def _as_scratch(output_split: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     if output_split is None or not output_split.is_contiguous():
         return None
