@@ -147,7 +147,11 @@ def test_append_then_decode_equals_attention_over_the_grown_cache(cuda_device):
     lens_t = torch.tensor(lens, dtype=torch.int32, device=dev)
     q_out = tda.qk_norm_rope_update_kvcache(qkv.to(dev), kd, vd, td, lens_t, wq.to(dev), wk.to(dev), cos.to(dev), sin.to(dev))
     out, lse = tda.flash_decode(q_out[:, 0], kd, vd, td, lens_t, d ** -0.5)
+    # the same through the mega-kernel builder's layout ([B, 1, Hq, D] in and out, default scale)
+    out4 = torch.full((len(lens), 1, hq, d), float("nan"), dtype=torch.bfloat16, device=dev)
+    assert tda.flash_decode_bsnh(q_out, kd, vd, td, lens_t, out4).data_ptr() == out4.data_ptr()
     torch.cuda.synchronize()
+    assert torch.equal(out4[:, 0], out)
     o64, l64 = cf.attn_fp64(q_ref[:, 0], k_ref, v_ref, table, lens, d ** -0.5)
     torch.testing.assert_close(out.double().cpu(), o64, atol=1e-2, rtol=2e-2)
     torch.testing.assert_close(lse.double().cpu(), l64, atol=2e-2, rtol=0)     # q rows may differ by a 16-bit rounding step

@@ -441,6 +441,32 @@ def inter_rank_combine(all_ranks_output: torch.Tensor, global_kv_lens: torch.Ten
     return final_output
 
 
+def flash_decode_bsnh(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                      block_tables: torch.Tensor, kv_lens: torch.Tensor, output: Optional[torch.Tensor] = None,
+                      sm_scale: Optional[float] = None, soft_cap: float = 0.0, stream=None) -> torch.Tensor:
+    """Decode in the layout of the reference's mega-kernel builder: argument order of
+    ``ModelBuilder.make_flash_decode`` (mega_triton_kernel/models/model_builder.py:248-286), which records an
+    ``attn_split`` + ``attn_combine`` task pair; this runs at once.
+
+    query / output ``[B, 1, Hq, D]`` (one new token per sequence, :274), caches ``[num_pages, P, Hkv, D]``,
+    ``sm_scale`` defaults to ``D ** -0.5`` (:275-276).  ``soft_cap`` is honoured (the builder zeroes it, :277)."""
+    if query.dim() != 4 or query.shape[1] != 1:
+        raise ValueError("query must be [B, 1, Hq, D]: flash decoding takes one query token per sequence")
+    batch, _, q_heads, d = query.shape
+    if output is None:
+        output = torch.empty((batch, 1, q_heads, d), dtype=query.dtype, device=query.device)
+    elif tuple(output.shape) != (batch, 1, q_heads, d):
+        raise ValueError(f"output must be [B, 1, Hq, D] = {(batch, 1, q_heads, d)}")
+    if sm_scale is None:
+        sm_scale = d ** -0.5
+    if query.is_cuda:
+        stream = _stream_handle(stream)
+    call = prepare_decode(query[:, 0], key_cache, value_cache, block_tables, kv_lens, sm_scale, soft_cap=soft_cap,
+                          out=output[:, 0], want_lse=False, work_queue=False)
+    call.run(stream)
+    return output
+
+
 def qk_norm_rope_update_kvcache(qkv: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
                                 block_tables: torch.Tensor, kv_lens: torch.Tensor, q_rms_weight: torch.Tensor,
                                 k_rms_weight: torch.Tensor, cos_cache: torch.Tensor, sin_cache: torch.Tensor,
