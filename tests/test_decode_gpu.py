@@ -578,6 +578,54 @@ def test_balanced_mode_many_sequences(cuda_device):
     _check(out[live], lse[live], q[live], k, v, table[live], [lens[i] for i in live], d ** -0.5, tag="balanced b150")
 
 
+def test_sequence_parallel_layer_mirror(cuda_device):
+    # the reference's layer (sp_flash_decode_layer.py:83-185) on one GPU: R layer objects stand in for R ranks, the
+    # exchange between them is a stack of their blocks
+    r_, b, hq, hkv, d, page = 3, 4, 32, 8, 128, 16
+    g = torch.Generator().manual_seed(19)
+    shard_lens = torch.tensor([[700, 16, 0, 33], [300, 0, 0, 1], [1, 77, 0, 2000]], dtype=torch.int32)
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    pool = 4 * 130
+    ks = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
+    vs = [torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device) for _ in range(r_)]
+    tables = [torch.randperm(pool, generator=g)[:b * 126].view(b, 126).to(torch.int32).to(cuda_device) for _ in range(r_)]
+    gl = shard_lens.to(cuda_device)
+    blocks = {}
+
+    def gather_for(rank):
+        def all_gather(block):
+            blocks[rank] = block
+            return torch.stack([blocks[i] for i in range(r_)]) if len(blocks) == r_ else None
+        return all_gather
+
+    layers = [tda.SpGQAFlashDecodeAttention(rk, 0, r_, 1, hq, hkv, d, d, page_size=page, scale=d ** -0.5,
+                                            max_allowed_batch=b, all_gather=gather_for(rk)) for rk in range(r_)]
+    for rk in range(r_ - 1):                       # the first ranks only deposit their block
+        blocks[rk] = layers[rk].local_decode(q, ks[rk], vs[rk], gl, tables[rk])
+    final = layers[r_ - 1](q, ks[r_ - 1], vs[r_ - 1], gl, tables[r_ - 1])
+    torch.cuda.synchronize()
+    assert final.shape == (b, hq, d) and final.dtype == torch.bfloat16
+    for i in range(b):
+        total = int(shard_lens[:, i].sum())
+        if total == 0:
+            assert (final[i] == 0).all()            # no rank holds tokens: defined as zero
+            continue
+        kk = torch.cat([cf.gather_kv(ks[rk], tables[rk][i].cpu(), int(shard_lens[rk, i])) for rk in range(r_)])
+        vv = torch.cat([cf.gather_kv(vs[rk], tables[rk][i].cpu(), int(shard_lens[rk, i])) for rk in range(r_)])
+        o64, _ = cf.attn_fp64(q[i:i + 1], kk[:, None].contiguous(), vv[:, None].contiguous(),
+                              torch.arange(total, dtype=torch.int32)[None], [total], d ** -0.5)
+        torch.testing.assert_close(final[i].double(), o64[0], atol=2e-2, rtol=2e-2)   # blocks travel in bf16
+    # one rank: forward needs no exchange and equals the plain decode
+    solo = tda.SpGQAFlashDecodeAttention(0, 0, 1, 1, hq, hkv, d, d, page_size=page, scale=d ** -0.5, max_allowed_batch=b)
+    got = solo(q, ks[0], vs[0], gl[:1], tables[0])
+    want, _ = tda.flash_decode(q, ks[0], vs[0], tables[0], gl[0], d ** -0.5)
+    torch.cuda.synchronize()
+    live = (shard_lens[0] > 0).to(cuda_device)
+    torch.testing.assert_close(got[live].float(), want[live].float(), atol=1e-2, rtol=1e-2)
+    with pytest.raises(ValueError):
+        tda.SpGQAFlashDecodeAttention(0, 0, 2, 1, hq, hkv, d, d)            # more ranks need an exchange
+
+
 @pytest.mark.parametrize("page", [6, 24])
 @pytest.mark.parametrize("algo", ["valu", "mfma"])
 def test_page_sizes_that_are_not_powers_of_two(cuda_device, page, algo):

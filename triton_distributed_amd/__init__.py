@@ -15,15 +15,28 @@ __all__ = [
 ]
 
 
+_LAYERS = ("SpGQAFlashDecodeAttention",)
+
+
+def _bind():
+    """Import the entry points (loads libfdk.so; raises if it is missing) and bind them on the package: the
+    function ``flash_decode`` takes the place of the submodule attribute of the same name that the import sets."""
+    mod = importlib.import_module(".flash_decode", __name__)
+    globals().update({n: getattr(mod, n) for n in __all__})
+
+
 def __getattr__(name):
+    if name in _LAYERS:
+        _bind()
+        mod = importlib.import_module(".sp_flash_decode_layer", __name__)
+        _bind()                                   # the layer module imports the submodule again
+        globals()[name] = getattr(mod, name)
+        return globals()[name]
     if name in __all__:
-        mod = importlib.import_module(".flash_decode", __name__)     # loads libfdk.so; raises if it is missing
-        # bind every entry point on the package (the function ``flash_decode`` takes the place of the
-        # submodule attribute of the same name that the import just set)
-        globals().update({n: getattr(mod, n) for n in __all__})
+        _bind()
         return globals()[name]
     raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
 
 
 def __dir__():
-    return sorted(list(globals()) + __all__)
+    return sorted(list(globals()) + __all__ + list(_LAYERS))
