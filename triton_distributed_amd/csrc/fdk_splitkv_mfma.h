@@ -568,7 +568,7 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     p.head_tiles = (p.group + 15) / 16;
     if (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) p.hg_per_wg = 1;
     p.hg_blocks = p.hkv / p.hg_per_wg;
-    const int nw = p.hg_per_wg > 4 ? p.hg_per_wg : 4;
+    const int nw = p.hg_per_wg >= 4 ? 8 : 4;      // wavefronts per workgroup (see mfma_kv_heads_per_wg)
     const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float)) + 16;
     constexpr int RPL = Regs<FP8, D>::RPL;
     int pm;
