@@ -2,7 +2,7 @@
 
 Tolerances (the bar this path is held to):
   out  bf16/fp16: |out - ref| <= 2e-2 + 2e-2*|ref| against the torch restatement of the reference's
-       torch implementation, and a tighter 5e-3 + 1e-2*|x| against the exact float64 answer;
+       torch implementation, and a tighter 8e-3 + 1e-2*|x| against the exact float64 answer;
   lse  fp32: |lse - lse64| <= 1e-3;
   block_table indexing: bit-exact where the mathematics allows it (single-token sequences, page
   permutations), no NaN/inf anywhere for kv_len >= 1."""
@@ -47,7 +47,9 @@ def _check(out, lse, q, k, v, table, lens, scale, soft_cap=0.0, k_scale=None, v_
     ref = ref_paged_attn(q, rk, rv, lens, table, scale, soft_cap)
     torch.testing.assert_close(out.float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL, msg=lambda m: f"{tag} vs torch ref: {m}")
     o64, l64 = cf.attn_fp64(q, rk, rv, table, lens, scale, soft_cap)
-    torch.testing.assert_close(out.double(), o64, atol=5e-3, rtol=1e-2, msg=lambda m: f"{tag} vs fp64: {m}")
+    # (P is rounded to the 16-bit dtype before the second product, as in the reference: with |v| ~ 3 a single
+    # element can be off by 6e-3 from the exact answer)
+    torch.testing.assert_close(out.double(), o64, atol=8e-3, rtol=1e-2, msg=lambda m: f"{tag} vs fp64: {m}")
     torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0, msg=lambda m: f"{tag} lse: {m}")
 
 
@@ -485,6 +487,53 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
     # against the oracle's restatement of the reference merge
     want = cf.combine_ranks(outs.cpu(), lses.cpu(), shard_lens)
     torch.testing.assert_close(final2.double().cpu(), want, atol=4e-3, rtol=1e-2)
+
+
+# ---- large batches: single pass with blocks of 4 or 8 kv heads per (eight-wave) workgroup ------------------------------
+@pytest.mark.parametrize("heads,batch,want_nh", [((32, 8), 256, 8), ((32, 8), 128, 4), ((16, 4), 256, 4), ((48, 2), 300, 2),
+                                                ((8, 8), 300, 8), ((96, 4), 130, 4)])
+@pytest.mark.parametrize("d,dtype,fp8,page", [(128, torch.bfloat16, False, 16), (128, torch.float16, False, 1),
+                                             (128, torch.bfloat16, True, 16), (64, torch.bfloat16, False, 6),
+                                             (256, torch.float16, False, 16), (256, torch.bfloat16, True, 64)])
+def test_large_batches_take_wide_head_blocks(cuda_device, heads, batch, want_nh, d, dtype, fp8, page):
+    hq, hkv = heads
+    print(f"case wide blocks heads={heads} B={batch} D={d} {dtype} fp8={fp8} P={page}", flush=True)
+    g = torch.Generator().manual_seed(batch * 7 + d + page)
+    lens = torch.randint(0, 150, (batch,), generator=g).tolist()
+    lens[0], lens[1], lens[batch - 1] = 149, 0, 1
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 2
+    q = torch.randn(batch, hq, d, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, max(pages) + 1), -7, dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t)
+    assert plan.num_splits == 1 and plan.kv_heads_per_wg == want_nh, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    empty = [i for i, n in enumerate(lens) if n == 0]
+    assert (out[empty] == 0).all() and (lse[empty] == float("-inf")).all()
+    rows = [i for i, n in enumerate(lens) if n > 0][:: max(1, batch // 24)] + [batch - 1]
+    _check(out[rows], lse[rows], q[rows], k, v, table[rows], [lens[i] for i in rows], d ** -0.5, ref_kv=ref_kv,
+           tag=f"wide blocks nh={want_nh}")
+    # the same call with the head block forced apart (a split count forces chunk mode with narrower blocks)
+    out2, lse2 = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, kv_split=2)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    torch.testing.assert_close(out[live].float(), out2[live].float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse[live], lse2[live], atol=1e-4, rtol=0)
 
 
 # ---- balanced mode: the kernel cuts the batch's KV ranges into equal shares from kv_lens ---------------------------
