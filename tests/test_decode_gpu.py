@@ -452,6 +452,57 @@ def test_hip_graph_replays_follow_the_inputs(cuda_device, mode):
                tag=f"graph replay {i}")
 
 
+def test_concurrent_host_threads_on_their_own_streams(cuda_device):
+    # The library keeps no mutable state apart from a thread-local error string: four host threads, each with its
+    # own stream, buffers and problem, call it at the same time (ctypes releases the GIL during the calls).
+    import threading
+    g = torch.Generator().manual_seed(71)
+    problems = []
+    for i, (b, hq, hkv, n, split) in enumerate([(3, 32, 8, 900, -1), (40, 32, 8, 300, -1), (2, 8, 1, 5000, 16), (5, 64, 8, 700, 3)]):
+        page, d = 16, 128
+        pages = (n + page - 1) // page
+        q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        k = torch.randn(b * pages, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        v = torch.randn(b * pages, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        table = torch.randperm(b * pages, generator=g).to(torch.int32).view(b, pages).to(cuda_device)
+        lens = torch.randint(1, n + 1, (b,), generator=g).to(torch.int32).to(cuda_device)
+        want = tda.flash_decode(q, k, v, table, lens, d ** -0.5, kv_split=split)
+        problems.append((q, k, v, table, lens, d ** -0.5, split, want))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(idx):
+        try:
+            q, k, v, table, lens, scale, split, want = problems[idx]
+            stream = torch.cuda.Stream(device=cuda_device)
+            call = tda.prepare_decode(q, k, v, table, lens, scale, kv_split=split)
+            for it in range(40):
+                call.out.fill_(float("nan"))
+                with torch.cuda.stream(stream):
+                    call.out.record_stream(stream)
+                    stream.wait_stream(torch.cuda.current_stream())
+                    out, lse = call.run(stream)
+                stream.synchronize()
+                if not (torch.equal(out, want[0]) and torch.equal(lse, want[1])):
+                    errors.append((idx, it))
+                    return
+            try:                                                  # a rejected call in one thread disturbs no other
+                tda.flash_decode(q, k, v, table.long(), lens, scale)
+                errors.append((idx, "int64 table accepted"))
+            except ValueError:
+                pass
+        except Exception as exc:                                  # noqa: BLE001
+            errors.append((idx, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(problems))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 def test_inter_rank_combine_equals_one_shot(cuda_device):
     # R ranks each hold a disjoint slice of every sequence (sequence parallel decode, one GPU stands in for all):
     # local decode per rank -> packed [R,B,Hq,D+1] -> merge == decode over the whole sequence

@@ -11,7 +11,6 @@ namespace fdk {
 constexpr int kHeadDim = 128;       // head dimension of the vector path (the matrix-core path: 64, 128, 256)
 constexpr int kWaveSize = 64;
 constexpr int kBalanceGranule = 64;  // tokens per unit of the balanced partition (a multiple of the 16-token tile)
-constexpr int kWavesPerWg = 4;      // split kernels run 256-thread workgroups
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

@@ -3,12 +3,13 @@
 //
 // Same contract as the vector-ALU kernel (fdk_splitkv_valu.h) and the same counterpart in the reference
 // (kernel_gqa_fwd_batch_decode_split_kv, python/triton_dist/kernels/nvidia/flash_decode.py:129-239, which
-// pads the q-head group to a 16-row tile for its tl.dot, :170-176).  One workgroup per (sequence, split,
-// block of kv heads, tile of 16 q heads).  Each wavefront owns one kv head; a workgroup covers up to eight
-// adjacent kv heads, so that together its wavefronts stream whole token rows (all heads of a token are
-// adjacent in the cache) - a compute unit then reads contiguous memory, which is worth ~8% of bandwidth
-// over eight workgroups reading one head each.  With fewer kv heads than wavefronts, the wavefronts of a
-// head interleave 16-token tiles and are merged through LDS at the end.
+// pads the q-head group to a 16-row tile for its tl.dot, :170-176).  A workgroup of four or eight wavefronts
+// works on pieces: a token range of one sequence for a block of 1, 2, 4 or 8 adjacent kv heads and a tile of 16
+// q heads.  Each wavefront owns one kv head; the wavefronts of a workgroup together stream runs of adjacent
+// heads of every token (all heads of a token are adjacent in the cache), which is worth ~8% of bandwidth over
+// workgroups reading one head each.  With fewer kv heads than wavefronts, the wavefronts of a head interleave
+// 16-token tiles and are merged through LDS at the end.  How pieces are handed out (one per workgroup, from a
+// queue, or as equal shares of the whole batch) is described at the end of the kernel.
 //
 // Per tile and wavefront:
 //   global -> registers   coalesced 16-byte loads, each instruction reads whole cache rows (head_dim 128: four
