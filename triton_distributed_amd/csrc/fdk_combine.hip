@@ -100,10 +100,26 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + wave;   // b * Hq + h
     if (row >= (int64_t)p.batch * p.hq) return;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
+    // The first kPre partial rows are requested before anything that depends on kv_lens is known (chunk mode:
+    // their addresses follow from (b, h) alone; rows past the live ones hold stale but readable workspace and
+    // are never used) - the kernel is a chain of dependent memory round trips, this removes one or two.
+    constexpr int kPre = 8;
+    float pre[kPre][EPL];
+    if (!p.balanced) {
+        const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
+#pragma unroll
+        for (int j = 0; j < kPre; ++j)
+            if (j < p.num_splits) Vec<EPL>::load(o_early + (int64_t)j * D, pre[j]);
+    }
     const PartRows pr = locate_rows<D>(p, b, h);
     const int live = pr.live;
     const float* lse_row = pr.lse;
     const float* o_row = pr.o + EPL * lane;
+    if (p.balanced) {
+#pragma unroll
+        for (int j = 0; j < kPre; ++j)
+            if (j < live) Vec<EPL>::load(o_row + j * pr.o_step, pre[j]);
+    }
 
     float m_run = -INFINITY, l_run = 0.f;
     float acc[EPL];
@@ -120,8 +136,20 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
         l_run = l_run * alpha + wave_sum(w);
 #pragma unroll
         for (int e = 0; e < EPL; ++e) acc[e] *= alpha;
+        int s = 0;
+        if (s0 == 0) {
+#pragma unroll
+            for (int j = 0; j < kPre; ++j) {
+                if (j < n) {
+                    const float ws = __shfl(w, j, 64);
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) acc[e] += ws * pre[j][e];
+                }
+            }
+            s = kPre;
+        }
 #pragma unroll 4
-        for (int s = 0; s < n; ++s) {
+        for (; s < n; ++s) {
             const float ws = __shfl(w, s, 64);
             float o[EPL];
             Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
@@ -155,14 +183,30 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     const int wave = threadIdx.x >> 6;
     const int64_t row = blockIdx.x;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
+    // as in combine_kernel: the first kPre rows of this wavefront (s = wave, wave + 4, ...) are requested early
+    constexpr int kPre = 8;
+    float pre[kPre][EPL];
+    if (!p.balanced) {
+        const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
+#pragma unroll
+        for (int j = 0; j < kPre; ++j)
+            if (wave + kRowsPerWg * j < p.num_splits) Vec<EPL>::load(o_early + (int64_t)(wave + kRowsPerWg * j) * D, pre[j]);
+    }
     const PartRows pr = locate_rows<D>(p, b, h);
     const int live = pr.live;
     const float* lse_row = pr.lse;
     const float* o_row = pr.o + EPL * lane;
+    if (p.balanced) {
+#pragma unroll
+        for (int j = 0; j < kPre; ++j)
+            if (wave + kRowsPerWg * j < live) Vec<EPL>::load(o_row + (wave + kRowsPerWg * j) * pr.o_step, pre[j]);
+    }
 
     float m = -INFINITY;
+    float my_first = -INFINITY;                    // lse of split `lane`, kept for the second pass
     for (int s0 = 0; s0 < live; s0 += 64) {
         const float my = s0 + lane < live ? lse_row[(s0 + lane) * pr.lse_step] : -INFINITY;
+        if (s0 == 0) my_first = my;
         m = fmaxf(m, wave_max(my));
     }
     m *= kLog2e;
@@ -172,10 +216,23 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
     for (int s0 = 0; s0 < live; s0 += 64) {
         const int n = min(64, live - s0);
-        const float w = lane < n ? fast_exp2(lse_row[(s0 + lane) * pr.lse_step] * kLog2e - m) : 0.f;
+        const float lse_s = s0 == 0 ? my_first : (lane < n ? lse_row[(s0 + lane) * pr.lse_step] : -INFINITY);
+        const float w = lane < n ? fast_exp2(lse_s * kLog2e - m) : 0.f;
         l += wave_sum(w);
+        int s = wave;
+        if (s0 == 0) {
+#pragma unroll
+            for (int j = 0; j < kPre; ++j) {
+                if (wave + kRowsPerWg * j < n) {
+                    const float ws = __shfl(w, wave + kRowsPerWg * j, 64);
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) acc[e] += ws * pre[j][e];
+                }
+            }
+            s = wave + kRowsPerWg * kPre;
+        }
 #pragma unroll 8
-        for (int s = wave; s < n; s += kRowsPerWg) {
+        for (; s < n; s += kRowsPerWg) {
             const float ws = __shfl(w, s, 64);
             float o[EPL];
             Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
