@@ -187,9 +187,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // account: the kernel cuts the KV ranges of the whole batch, as kv_lens gives them, into equal shares, so
     // that a ragged batch loads every workgroup alike.  The workspace then holds (shares + batch) slots of
     // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
-    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && splits > 1 && batch <= kMaxBalancedBatch) {
+    const int64_t columns = (int64_t)batch * cdiv64(max_len, fdk::kBalanceGranule);   // granules of all sequences, at most
+    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && splits > 1 && batch <= kMaxBalancedBatch &&
+        columns < (1 << 30)) {                                            // the kernel counts granules in int32
         const int64_t gran = fdk::kBalanceGranule;
-        const int64_t columns = (int64_t)batch * cdiv64(max_len, gran);      // granules of all sequences, at most
         int64_t shares = columns / (min_chunk / gran);
         const int64_t most = 2 * (int64_t)num_cus / units_per_seq;           // two workgroups per compute unit
         if (shares > most) shares = most;
