@@ -647,6 +647,42 @@ def test_balanced_mode_ragged_batches(cuda_device, name):
     torch.testing.assert_close(lse[live], lse_c[live], atol=1e-4, rtol=0)
 
 
+def test_balanced_mode_with_soft_cap_strides_and_output_forms(cuda_device):
+    # fp16, soft cap, q / out taken as strided views, fp32 output, packed [B, Hq, D+1] output - all in balanced mode
+    g = torch.Generator().manual_seed(83)
+    lens, hq, hkv, d, page = [30000, 11, 17000], 16, 2, 128, 16
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 1
+    q_big = torch.randn(3, hq, 2 * d, generator=g).to(torch.float16).to(cuda_device)
+    q = q_big[:, :, :d]                                           # head stride 2 D, contiguous D
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    table = torch.zeros((3, max(pages)), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    scale, cap = d ** -0.5, 30.0
+    assert tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens)).balanced
+    out32 = torch.full((3, hq, d + 3), float("nan"), dtype=torch.float32, device=cuda_device)
+    o, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), out=out32[:, :, :d])
+    packed = torch.full((3, hq, d + 1), float("nan"), dtype=torch.float16, device=cuda_device)
+    tda.prepare_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), packed_out=packed,
+                       want_lse=False).run()
+    torch.cuda.synchronize()
+    assert o.data_ptr() == out32.data_ptr() and torch.isnan(out32[:, :, d:]).all()      # nothing written past D
+    o64, l64 = cf.attn_fp64(q, k, v, table, lens, scale, cap)
+    torch.testing.assert_close(o.double(), o64, atol=8e-3, rtol=1e-2)
+    torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0)
+    torch.testing.assert_close(packed[..., :d].float(), o, atol=2e-3, rtol=2e-3)        # fp16 rounding of the same result
+    torch.testing.assert_close(packed[..., d].float(), lse, atol=1e-2, rtol=1e-3)
+    ref = ref_paged_attn(q, k, v, lens, table, scale, cap)
+    torch.testing.assert_close(packed[..., :d].float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL)
+
+
 def test_balanced_mode_many_sequences(cuda_device):
     # more than 64 sequences: the partition scan runs over several 64-lane chunks; includes empty sequences
     g = torch.Generator().manual_seed(77)
