@@ -338,6 +338,30 @@ def test_split_invariance(cuda_device):
         torch.testing.assert_close(res[s][1], res[1][1], atol=2e-5, rtol=0)
 
 
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+@pytest.mark.parametrize("kv_split", [-1, 1, 4])
+def test_a_length_hint_that_is_too_small_loses_no_tokens(cuda_device, algo, kv_split):
+    # max_kv_len only sizes the plan: the last split runs to the end of each sequence
+    g = torch.Generator().manual_seed(91)
+    lens, hq, hkv, d, page = [1000, 37, 2500, 640], 32, 8, 128, 16
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages)
+    q = torch.randn(4, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.zeros((4, max(pages)), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5, max_kv_len=600, kv_split=kv_split,
+                                algo=algo)
+    torch.cuda.synchronize()
+    _check(out, lse, q, k, v, table, lens, d ** -0.5, tag=f"small hint {algo} S={kv_split}")
+
+
 def test_zero_length_sequence_is_defined(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=300), cuda_device)
     lens = _lens_t([300, 0, 17], cuda_device)

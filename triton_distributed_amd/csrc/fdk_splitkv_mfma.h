@@ -460,7 +460,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         wg /= p.hg_blocks;
         const int split = wg % p.num_splits;
         const int pb = wg / p.num_splits;
-        run_piece(pb, hgb, ht, split * p.chunk, split * p.chunk + p.chunk,
+        // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
+        run_piece(pb, hgb, ht, split * p.chunk, split == p.num_splits - 1 ? p.max_tokens : split * p.chunk + p.chunk,
                   ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split, p.num_splits);
         return;
     }
@@ -520,7 +521,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const int split = wg % p.num_splits;
             pb = wg / p.num_splits;
             c_start = split * p.chunk;
-            c_limit = c_start + p.chunk;
+            c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + p.chunk;
             prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
             prow_step = p.num_splits;
         }

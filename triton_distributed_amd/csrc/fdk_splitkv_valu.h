@@ -111,7 +111,8 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
         }
         return;
     }
-    const int c_end = min(c_start + p.chunk, kv_len);
+    // the last split runs to the end of the sequence (see the matrix-core kernel)
+    const int c_end = split == p.num_splits - 1 ? kv_len : min(c_start + p.chunk, kv_len);
     const int tile_tokens = NJ * ti_n * TPL;        // tokens one workgroup tile covers
     const int n_full = (c_end - c_start) / tile_tokens;
     const bool has_tail = (c_end - c_start) % tile_tokens != 0;
