@@ -44,3 +44,28 @@ def test_tiny_config_shapes():
     assert tuple(c["q"].shape) == (2, 8, 128) and tuple(c["k_cache"].shape) == (1024, 1, 2, 128)
     assert sorted(c["block_table"].flatten().tolist()) == list(range(1024))      # a permutation of the pool
     assert GOLDEN["tiny.out64"].shape == (2, 8, 128) and GOLDEN["tiny.lse64"].shape == (2, 8)
+
+
+# ---- the RMSNorm + rotary + paged-append operator -----------------------------------------------------------------
+from cases_kv_append import KV_APPEND_CASES, as_f32, kv_append_case  # noqa: E402
+from oracle import kv_append as okv  # noqa: E402
+
+KV_GOLDEN = np.load(os.path.join(ROOT, "tests", "golden", "kv_append_golden.npz"))
+
+
+@pytest.mark.parametrize("name", list(KV_APPEND_CASES))
+def test_kv_append_oracle_reproduces_golden(name):
+    c = kv_append_case(name)
+    assert abs(float(c["qkv"].double().sum()) - float(KV_GOLDEN[name + ".qkv_sum"])) < 1e-9
+    cos, sin = okv.cos_sin_tables(c["qkv"].shape[-1], c["max_positions"], c["rope_theta"])
+    q_out = okv.kv_append(c["qkv"], c["k"], c["v"], c["table"], c["lens"], c["wq"], c["wk"], cos, sin, c["hq"],
+                          k_scale=c["k_scale"], v_scale=c["v_scale"])
+    step = 2.0 ** -7 if c["qkv"].dtype == torch.bfloat16 else 2.0 ** -10
+    # torch's CPU reductions may differ in the last fp32 bit between builds: at most one 16-bit rounding step
+    # (for a rotated element: of its pair's magnitude; for an fp8 byte: one e4m3 code = 2^-3)
+    pair = np.abs(KV_GOLDEN[name + ".q_out"]).max()
+    np.testing.assert_allclose(as_f32(q_out), KV_GOLDEN[name + ".q_out"], rtol=step, atol=2.5 * step * pair)
+    k_step = 2.0 ** -3 if c["k"].dtype == torch.float8_e4m3fn else step
+    np.testing.assert_allclose(as_f32(c["k"]), KV_GOLDEN[name + ".k"], rtol=k_step, atol=2.5 * k_step * np.abs(KV_GOLDEN[name + ".k"]).max())
+    np.testing.assert_array_equal(as_f32(c["v"]), KV_GOLDEN[name + ".v"])              # copies / exact quotients
+    assert (as_f32(q_out) == KV_GOLDEN[name + ".q_out"]).mean() > 0.99                 # and in fact (almost) all equal

@@ -11,13 +11,17 @@ import pytest
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
 
 import triton_distributed_amd as tda  # noqa: E402
 from oracle import closed_form as cf  # noqa: E402
 from oracle import fp8 as ofp8  # noqa: E402
 from oracle import kv_append as okv  # noqa: E402
 
+from cases_kv_append import KV_APPEND_CASES, as_f32, kv_append_case  # noqa: E402
+
 pytestmark = pytest.mark.gpu
+KV_GOLDEN = __import__("numpy").load(os.path.join(ROOT, "tests", "golden", "kv_append_golden.npz"))
 
 
 def _setup(seed, lens, t, hq, hkv, d, page, dtype, spare=3, theta=1000000.0, poison=True):
@@ -85,6 +89,28 @@ def test_append_matches_the_oracle(cuda_device, d, dtype, page, t):
             for h in (0, hq - 1):
                 want = okv.norm_rope_fp64(qkv[b, j, h], wq, 1e-6, pos)
                 torch.testing.assert_close(q_out[b, j, h].cpu().double(), want, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("name", list(KV_APPEND_CASES))
+def test_append_matches_the_committed_vectors(cuda_device, name):
+    c = kv_append_case(name)
+    dev = cuda_device
+    cos, sin = okv.cos_sin_tables(c["qkv"].shape[-1], c["max_positions"], c["rope_theta"])
+    kd, vd = c["k"].to(dev), c["v"].to(dev)
+    sc = {} if c["k_scale"] is None else dict(k_scale=c["k_scale"].to(dev), v_scale=c["v_scale"].to(dev))
+    q_out = tda.qk_norm_rope_update_kvcache(c["qkv"].to(dev), kd, vd, c["table"].to(dev),
+                                            torch.tensor(c["lens"], dtype=torch.int32, device=dev), c["wq"].to(dev),
+                                            c["wk"].to(dev), cos.to(dev), sin.to(dev), **sc)
+    torch.cuda.synchronize()
+    dtype = c["qkv"].dtype
+    _ulp_close(q_out.float().cpu(), torch.from_numpy(KV_GOLDEN[name + ".q_out"]), dtype, "q_out vs golden")
+    assert (as_f32(vd.cpu()) == KV_GOLDEN[name + ".v"]).all()
+    if c["k_scale"] is None:
+        _ulp_close(kd.float().cpu(), torch.from_numpy(KV_GOLDEN[name + ".k"]), dtype, "k vs golden")
+    else:
+        got, want = torch.from_numpy(as_f32(kd.cpu())), torch.from_numpy(KV_GOLDEN[name + ".k"])
+        assert ((got - want).abs() <= 0.126 * torch.maximum(got.abs(), want.abs()) + 2.0 ** -9).all()
+        assert (got != want).float().mean() < 0.02
 
 
 def test_positions_outside_the_table_and_poisoned_entries_are_not_written(cuda_device):
