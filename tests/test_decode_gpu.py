@@ -372,6 +372,46 @@ def test_zero_length_sequence_is_defined(cuda_device):
         assert torch.isfinite(out[0].float()).all() and torch.isfinite(lse[[0, 2]]).all()
 
 
+@pytest.mark.parametrize("algo", ["valu", "mfma"])
+def test_lengths_outside_the_table_are_clamped_and_negative_ones_are_empty(cuda_device, algo):
+    # kv_lens is device data the host never sees: a length beyond the table attends the table's capacity, a
+    # negative one nothing - in every plan mode, without reading outside the table
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=4, kv_len=320), cuda_device)
+    cap = inp.block_table.shape[1] * 16
+    lens = _lens_t([cap + 5000, -3, 17, 2 ** 31 - 1], cuda_device)
+    for kw in (dict(kv_split=1), dict(kv_split=5), dict()):
+        out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, lens, inp.sm_scale, algo=algo, **kw)
+        torch.cuda.synchronize()
+        assert torch.all(out[1] == 0) and torch.all(torch.isneginf(lse[1]))
+        _check(out[[0, 2, 3]], lse[[0, 2, 3]], inp.q[[0, 2, 3]], inp.k_cache, inp.v_cache, inp.block_table[[0, 2, 3]],
+               [cap, 17, cap], inp.sm_scale, tag=f"clamped {algo} {kw}")
+
+
+def test_fp16_queries_with_an_fp8_cache(cuda_device):
+    g = torch.Generator().manual_seed(97)
+    lens, hq, hkv, d, page = [700, 3, 129, 2000], 32, 8, 128, 16
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 1
+    q = torch.randn(4, hq, d, generator=g).to(torch.float16).to(cuda_device)
+    k16 = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    v16 = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    table = torch.zeros((4, max(pages)), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    k8, ks = wl.quantize_kv_fp8(k16)
+    v8, vs = wl.quantize_kv_fp8(v16)
+    ref_kv = (ofp8.dequant_per_head(k8, ks, torch.float16), ofp8.dequant_per_head(v8, vs, torch.float16))
+    for kw in (dict(), dict(kv_split=6), dict(algo="valu")):
+        out, lse = tda.flash_decode(q, k8, v8, table, _lens_t(lens, cuda_device), d ** -0.5, k_scale=ks, v_scale=vs, **kw)
+        torch.cuda.synchronize()
+        assert out.dtype == torch.float16
+        _check(out, lse, q, k8, v8, table, lens, d ** -0.5, ref_kv=ref_kv, tag=f"fp16 q / fp8 kv {kw}")
+
+
 def test_split_then_combine_entry_points_equal_the_fused_call(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=4, kv_len=2048), cuda_device)
     for s in (1, 8):
