@@ -747,6 +747,28 @@ def test_balanced_mode_with_soft_cap_strides_and_output_forms(cuda_device):
     torch.testing.assert_close(packed[..., :d].float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL)
 
 
+def test_balanced_mode_clamps_lengths_like_the_other_modes(cuda_device):
+    g = torch.Generator().manual_seed(89)
+    hq, hkv, d, page, width = 8, 1, 128, 16, 2600
+    cap = width * page
+    true_lens = [cap, 0, 30000]                                   # what the device lengths below amount to
+    pool = width + 1875 + 2
+    q = torch.randn(3, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((3, width), -9, dtype=torch.int32)
+    table[0] = perm[:width]
+    table[2, :1875] = perm[width:width + 1875]
+    table = table.to(cuda_device)
+    lens_t = _lens_t([cap + 1000, -1, 30000], cuda_device)
+    assert tda.get_split_kv_plan(q, k, v, table, lens_t).balanced
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5)
+    torch.cuda.synchronize()
+    assert torch.all(out[1] == 0) and torch.all(torch.isneginf(lse[1]))
+    _check(out[[0, 2]], lse[[0, 2]], q[[0, 2]], k, v, table[[0, 2]], [cap, 30000], d ** -0.5, tag="balanced clamp")
+
+
 def test_balanced_mode_many_sequences(cuda_device):
     # more than 64 sequences: the partition scan runs over several 64-lane chunks; includes empty sequences
     g = torch.Generator().manual_seed(77)
