@@ -39,13 +39,16 @@ def _lens_t(lens, device):
     return torch.as_tensor(list(lens), dtype=torch.int32, device=device)
 
 
-def _check(out, lse, q, k, v, table, lens, scale, soft_cap=0.0, k_scale=None, v_scale=None, ref_kv=None, tag=""):
-    """Compare one result with both oracles (run on the tensors' own device)."""
+def _check(out, lse, q, k, v, table, lens, scale, soft_cap=0.0, k_scale=None, v_scale=None, ref_kv=None, tag="",
+           ref_tol=None):
+    """Compare one result with both oracles (run on the tensors' own device).  ``ref_tol`` widens the comparison with
+    the torch restatement only (it rounds its logits to 16 bits, so its own error grows with the logit scale)."""
     assert torch.isfinite(out.float()).all(), f"{tag}: non-finite out"
     assert torch.isfinite(lse).all(), f"{tag}: non-finite lse"
     rk, rv = ref_kv if ref_kv is not None else (k, v)
     ref = ref_paged_attn(q, rk, rv, lens, table, scale, soft_cap)
-    torch.testing.assert_close(out.float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL, msg=lambda m: f"{tag} vs torch ref: {m}")
+    torch.testing.assert_close(out.float(), ref.float(), atol=ref_tol or OUT_ATOL, rtol=ref_tol or OUT_RTOL,
+                               msg=lambda m: f"{tag} vs torch ref: {m}")
     o64, l64 = cf.attn_fp64(q, rk, rv, table, lens, scale, soft_cap)
     # (P is rounded to the 16-bit dtype before the second product, as in the reference: with |v| ~ 3 a single
     # element can be off by 6e-3 from the exact answer)
@@ -865,6 +868,64 @@ def test_page_sizes_that_are_not_powers_of_two(cuda_device, page, algo):
                                 c["sm_scale"], algo=algo)
     torch.cuda.synchronize()
     _check(out, lse, c["q"], c["k_cache"], c["v_cache"], c["block_table"], c["kv_lens"], c["sm_scale"], tag=f"P={page}")
+
+
+# ---- seeded random sweep over the whole argument space -------------------------------------------------------------
+@pytest.mark.parametrize("seed", list(range(96)))
+def test_random_shapes_against_the_oracle(cuda_device, seed):
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.choice([64, 128, 128, 256]))
+    hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    group = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 20]))
+    hq = hkv * group
+    page = int(rng.choice([1, 2, 3, 4, 8, 16, 16, 32, 64, 24]))
+    batch = int(rng.choice([1, 2, 5, 17, 40, 90]))
+    n_max = int(rng.choice([40, 300, 1500, 3000])) if batch <= 40 else int(rng.choice([40, 200]))
+    dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+    fp8 = bool(rng.random() < 0.25)
+    soft_cap = float(rng.choice([0.0, 0.0, 30.0]))
+    kv_split = int(rng.choice([-1, -1, -1, 1, 2, 5, 32]))
+    lens = rng.integers(0, n_max + 1, size=batch).tolist()
+    lens[int(rng.integers(0, batch))] = n_max
+    if rng.random() < 0.5:
+        lens[int(rng.integers(0, batch))] = 1
+    hint = None if rng.random() < 0.5 else int(n_max * rng.choice([0.5, 1.0, 2.0]))
+    print(f"case random seed={seed} B={batch} {hq}q/{hkv}kv D={d} P={page} N<={n_max} {dtype} fp8={fp8} cap={soft_cap} "
+          f"S={kv_split} hint={hint}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 3
+    q = torch.randn(batch, hq, d, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, max(max(pages), 1) + int(rng.integers(0, 3))), int(rng.choice([-1, 2 ** 31 - 1, 0])), dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
+    scale_mult = float(rng.choice([0.5, 1.0, 1.0, 2.0]))
+    scale = float(d ** -0.5) * scale_mult
+    if hint is not None and hint < max(lens):
+        hint_arg = hint                                # too small on purpose: costs balance, not tokens
+    else:
+        hint_arg = hint
+    out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), scale, soft_cap=soft_cap, kv_split=kv_split,
+                                max_kv_len=hint_arg, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    empty = [i for i, n in enumerate(lens) if n == 0]
+    live = [i for i, n in enumerate(lens) if n > 0]
+    if empty:
+        assert (out[empty] == 0).all() and torch.isneginf(lse[empty]).all()
+    # doubled logits double the 16-bit logit rounding of the torch restatement; the float64 comparison stays as tight
+    _check(out[live], lse[live], q[live], k, v, table[live], [lens[i] for i in live], scale, soft_cap, ref_kv=ref_kv,
+           tag=f"random seed {seed}", ref_tol=4e-2 if scale_mult > 1.0 else None)
 
 
 # ---- fp8 KV cache ------------------------------------------------------------------------------------------------
