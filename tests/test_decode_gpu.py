@@ -928,6 +928,68 @@ def test_random_shapes_against_the_oracle(cuda_device, seed):
            tag=f"random seed {seed}", ref_tol=4e-2 if scale_mult > 1.0 else None)
 
 
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_long_and_wide_batches_against_the_oracle(cuda_device, seed):
+    # the plans the small sweep above rarely reaches: balanced mode (few long sequences) and single pass with wide
+    # head blocks (many short sequences)
+    rng = np.random.default_rng(5000 + seed)
+    long_case = seed % 3 != 2
+    d = int(rng.choice([64, 128, 128, 256]))
+    page = int(rng.choice([1, 4, 16, 16, 64, 24]))
+    dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+    fp8 = bool(rng.random() < 0.3)
+    soft_cap = float(rng.choice([0.0, 0.0, 50.0]))
+    if long_case:
+        hkv = int(rng.choice([1, 2, 4]))
+        group = int(rng.choice([1, 4, 8, 16, 24]))
+        batch = int(rng.choice([1, 2, 3, 6]))
+        n_max = int(rng.choice([20000, 33000, 48000])) // (2 if d == 256 or hkv == 4 else 1)
+        lens = rng.integers(0, n_max + 1, size=batch).tolist()
+        lens[int(rng.integers(0, batch))] = n_max
+    else:
+        hkv = int(rng.choice([4, 8]))
+        group = int(rng.choice([1, 4, 8]))
+        batch = int(rng.choice([260, 300, 520]))
+        n_max = 70
+        lens = rng.integers(0, n_max + 1, size=batch).tolist()
+    hq = hkv * group
+    print(f"case random2 seed={seed} B={batch} {hq}q/{hkv}kv D={d} P={page} N<={n_max} {dtype} fp8={fp8} cap={soft_cap}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 2
+    q = torch.randn(batch, hq, d, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, max(max(pages), 1) + 1), -1, dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
+    scale = float(d ** -0.5)
+    lens_t = _lens_t(lens, cuda_device)
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=n_max)
+    if long_case:
+        assert plan.balanced or plan.num_splits > 1, plan
+    else:
+        assert plan.num_splits == 1 and plan.kv_heads_per_wg >= 2, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=soft_cap, max_kv_len=n_max, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    empty = [i for i, n in enumerate(lens) if n == 0]
+    live = [i for i, n in enumerate(lens) if n > 0]
+    if empty:
+        assert (out[empty] == 0).all() and torch.isneginf(lse[empty]).all()
+    rows = live if long_case else live[:: max(1, len(live) // 20)]
+    _check(out[rows], lse[rows], q[rows], k, v, table[rows], [lens[i] for i in rows], scale, soft_cap, ref_kv=ref_kv,
+           tag=f"random2 seed {seed} {plan}")
+
+
 # ---- fp8 KV cache ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("heads", [(32, 8), (64, 8), (8, 8)])
 @pytest.mark.parametrize("algo", ["valu", "mfma"])
