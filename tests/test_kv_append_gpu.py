@@ -113,6 +113,51 @@ def test_append_matches_the_committed_vectors(cuda_device, name):
         assert (got != want).float().mean() < 0.02
 
 
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_random_appends_against_the_oracle(cuda_device, seed):
+    import numpy as np
+    rng = np.random.default_rng(300 + seed)
+    d = int(rng.choice([64, 128, 256]))
+    dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+    page = int(rng.choice([1, 2, 3, 8, 16, 64]))
+    t = int(rng.choice([1, 1, 2, 7]))
+    hkv = int(rng.choice([1, 2, 8]))
+    hq = hkv * int(rng.choice([0, 1, 4, 5]))                      # 0: only the cache is updated
+    batch = int(rng.choice([1, 3, 9]))
+    lens = (rng.integers(0, 200, size=batch) + t).tolist()
+    fp8 = bool(rng.random() < 0.3) and dtype == torch.bfloat16
+    print(f"case random append seed={seed} B={batch} T={t} {hq}q/{hkv}kv D={d} P={page} {dtype} fp8={fp8}", flush=True)
+    qkv, wq, wk, table, k, v, cos, sin = _setup(seed, lens, t, hq, hkv, d, page, dtype, theta=float(rng.choice([1e4, 1e6])))
+    ks = vs = None
+    if fp8:
+        k = torch.zeros(k.shape, dtype=torch.float8_e4m3fn)
+        v = torch.zeros(v.shape, dtype=torch.float8_e4m3fn)
+        ks = torch.tensor(rng.uniform(0.01, 0.03, size=hkv), dtype=torch.float32)
+        vs = torch.tensor(rng.uniform(0.01, 0.03, size=hkv), dtype=torch.float32)
+    k_ref, v_ref = k.clone(), v.clone()
+    q_ref = okv.kv_append(qkv, k_ref, v_ref, table, lens, wq, wk, cos, sin, hq, 1e-5, 1e-6, k_scale=ks, v_scale=vs)
+    dev = cuda_device
+    kd, vd = k.to(dev), v.to(dev)
+    sc = {} if ks is None else dict(k_scale=ks.to(dev), v_scale=vs.to(dev))
+    q_out = tda.qk_norm_rope_update_kvcache(qkv.to(dev), kd, vd, table.to(dev),
+                                            torch.tensor(lens, dtype=torch.int32, device=dev), wq.to(dev), wk.to(dev),
+                                            cos.to(dev), sin.to(dev), None, 1e-5, 1e-6, **sc)
+    torch.cuda.synchronize()
+    if hq:
+        _ulp_close(q_out.cpu(), q_ref, dtype, "q_out")
+    else:
+        assert q_out.numel() == 0
+    if fp8:
+        tab = torch.from_numpy(ofp8.e4m3fn_table())
+        assert torch.equal(vd.cpu().view(torch.uint8), v_ref.view(torch.uint8))
+        got, want = tab[kd.cpu().view(torch.uint8).long()], tab[k_ref.view(torch.uint8).long()]
+        assert ((got - want).abs() <= 0.126 * torch.maximum(got.abs(), want.abs()) + 2.0 ** -9).all()
+        assert (got != want).float().mean() < 0.03
+    else:
+        assert torch.equal(vd.cpu(), v_ref)
+        _ulp_close(kd.cpu(), k_ref, dtype, "k_cache")
+
+
 def test_positions_outside_the_table_and_poisoned_entries_are_not_written(cuda_device):
     dev = cuda_device
     hq, hkv, d, page, t = 4, 2, 128, 16, 2
