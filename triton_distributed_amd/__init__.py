@@ -16,6 +16,7 @@ __all__ = [
 
 
 _LAYERS = ("SpGQAFlashDecodeAttention",)
+_HOST_ONLY = {"PagedKVCache": ".paged_kv_cache"}      # importable without the library
 
 
 def _bind():
@@ -26,6 +27,9 @@ def _bind():
 
 
 def __getattr__(name):
+    if name in _HOST_ONLY:
+        globals()[name] = getattr(importlib.import_module(_HOST_ONLY[name], __name__), name)
+        return globals()[name]
     if name in _LAYERS:
         _bind()
         mod = importlib.import_module(".sp_flash_decode_layer", __name__)
@@ -39,4 +43,4 @@ def __getattr__(name):
 
 
 def __dir__():
-    return sorted(list(globals()) + __all__ + list(_LAYERS))
+    return sorted(list(globals()) + __all__ + list(_LAYERS) + list(_HOST_ONLY))

@@ -1,0 +1,132 @@
+"""Paged KV cache of a decoder stack: the producer of the tensors the decode and append operators take.
+
+Host-side mirror of the reference's ``PagedKVCache`` (mega_triton_kernel/models/paged_kv_cache.py:28-58): one K
+pool and one V pool ``[num_blocks, PAGE_SIZE, Hkv, D]`` shared by all layers, ``block_tables
+[num_layers, B, max_blocks_per_seq]`` int32 cut from ONE permutation of the pool (no page belongs to two
+sequences or two layers), one ``kv_lens [B]`` int32 for all layers, ``inc_offset`` and ``get_layer_kv_cache``
+with the reference's meaning.
+
+Differences, all additions:
+  * the pools start zeroed (the reference fills them with random numbers), ``fill="randn"`` restores that;
+  * ``dtype=torch.float8_e4m3fn`` keeps 1-byte pools plus per-layer, per-kv-head fp32 scales
+    (``k_scale, v_scale [num_layers, Hkv]``, given by the caller);
+  * the lengths are tracked on the host as well (``max_kv_len``), so the decode can be planned for the real
+    length without reading ``kv_lens`` back from the GPU - a hint that is too small never drops tokens;
+  * ``append`` / ``decode`` run the two operators of this package on one layer's view.
+
+The class itself allocates with torch and launches nothing; it works on any torch device (the operators do not).
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+
+class PagedKVCache:
+
+    def __init__(self, PAGE_SIZE: int = 1, num_layers: int = 32, batch_size: int = 1, max_length: int = 1024,
+                 num_kv_heads: int = 8, head_dim: int = 128, dtype=torch.bfloat16, *, device=None,
+                 fill: str = "zeros", generator: Optional[torch.Generator] = None,
+                 k_scale: Optional[torch.Tensor] = None, v_scale: Optional[torch.Tensor] = None) -> None:
+        if PAGE_SIZE <= 0 or num_layers <= 0 or batch_size <= 0 or max_length <= 0:
+            raise ValueError("PAGE_SIZE, num_layers, batch_size and max_length must be positive")
+        if fill not in ("zeros", "randn"):
+            raise ValueError("fill must be 'zeros' or 'randn'")
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        self.device = torch.device(device)
+        self.page_size = PAGE_SIZE
+        self.max_num_blocks_per_seq = (max_length + PAGE_SIZE - 1) // PAGE_SIZE
+        self.num_layers = num_layers
+        self.batch_size = batch_size
+        self.max_length = max_length
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.dtype = dtype
+        num_blocks = self.max_num_blocks_per_seq * batch_size * num_layers
+        if num_blocks >= 2 ** 31:
+            raise ValueError("block ids are int32")
+        shape = (num_blocks, PAGE_SIZE, num_kv_heads, head_dim)
+        fp8 = dtype == torch.float8_e4m3fn
+        if fp8:
+            if k_scale is None or v_scale is None:
+                raise ValueError("an fp8 cache needs k_scale and v_scale [num_layers, Hkv]")
+            for s in (k_scale, v_scale):
+                if tuple(s.shape) != (num_layers, num_kv_heads) or s.dtype != torch.float32:
+                    raise ValueError("k_scale / v_scale must be fp32 [num_layers, Hkv]")
+            self.k_scale = k_scale.to(self.device).contiguous()
+            self.v_scale = v_scale.to(self.device).contiguous()
+        else:
+            self.k_scale = self.v_scale = None
+        if fill == "zeros":
+            self.key_cache = torch.zeros(shape, dtype=dtype, device=self.device)
+            self.value_cache = torch.zeros(shape, dtype=dtype, device=self.device)
+        else:
+            # drawn on the host so that a seed gives the same cache on every device
+            draw = torch.bfloat16 if fp8 else dtype
+            self.key_cache = torch.randn(shape, generator=generator, dtype=draw).to(dtype).to(self.device)
+            self.value_cache = torch.randn(shape, generator=generator, dtype=draw).to(dtype).to(self.device)
+        perm = torch.randperm(num_blocks, generator=generator).to(torch.int32)
+        self.block_tables = perm.reshape(num_layers, batch_size, self.max_num_blocks_per_seq).to(self.device)
+        self.kv_lens = torch.zeros(batch_size, dtype=torch.int32, device=self.device)
+        self._host_len = 0
+
+    # ---- the reference's interface -----------------------------------------------------------------------------
+    def inc_offset(self, seq_len: int) -> None:
+        """Every sequence grows by ``seq_len`` tokens (paged_kv_cache.py:52-54).  Call BEFORE appending them: the
+        append operator expects lengths that already count the new tokens."""
+        if seq_len < 0 or self._host_len + seq_len > self.max_length:
+            raise ValueError(f"{self._host_len} + {seq_len} tokens exceed max_length = {self.max_length}")
+        self.kv_lens += seq_len
+        self._host_len += seq_len
+
+    def get_layer_kv_cache(self, layer_idx: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+        """``(key_cache, value_cache, block_table [B, max_blocks_per_seq], kv_lens [B])`` of one layer
+        (paged_kv_cache.py:56-57); views, nothing is copied."""
+        return self.key_cache, self.value_cache, self.block_tables[layer_idx], self.kv_lens
+
+    # ---- additions ---------------------------------------------------------------------------------------------
+    @property
+    def max_kv_len(self) -> int:
+        """Length of every sequence as the host knows it (all sequences advance together)."""
+        return self._host_len
+
+    @property
+    def nbytes(self) -> int:
+        return 2 * self.key_cache.numel() * self.key_cache.element_size()
+
+    def reset(self) -> None:
+        """Forget all tokens; the pages keep their contents and their owners."""
+        self.kv_lens.zero_()
+        self._host_len = 0
+
+    def layer_scales(self, layer_idx: int):
+        if self.k_scale is None:
+            return None, None
+        return self.k_scale[layer_idx], self.v_scale[layer_idx]
+
+    def append(self, layer_idx: int, qkv: torch.Tensor, q_rms_weight: torch.Tensor, k_rms_weight: torch.Tensor,
+               cos_cache: torch.Tensor, sin_cache: torch.Tensor, q_rms_eps: float = 1e-6, k_rms_eps: float = 1e-6,
+               q_norm_rope: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+        """Norm + rotary + append of ``qkv [B, T, Hq + 2 Hkv, D]`` into one layer, after ``inc_offset(T)``.
+        Returns the normalised, rotated query ``[B, T, Hq, D]``."""
+        from . import qk_norm_rope_update_kvcache
+        if qkv.shape[1] > self._host_len:
+            raise ValueError("call inc_offset(T) before append: kv_lens must count the new tokens")
+        k, v, table, lens = self.get_layer_kv_cache(layer_idx)
+        ks, vs = self.layer_scales(layer_idx)
+        return qk_norm_rope_update_kvcache(qkv, k, v, table, lens, q_rms_weight, k_rms_weight, cos_cache, sin_cache,
+                                           q_norm_rope, q_rms_eps, k_rms_eps, k_scale=ks, v_scale=vs, stream=stream)
+
+    def decode(self, layer_idx: int, q: torch.Tensor, sm_scale: float, **kwargs):
+        """``flash_decode`` of ``q [B, Hq, D]`` over one layer, planned for the host-known length.
+        Returns ``(out [B, Hq, D], lse [B, Hq] fp32)``."""
+        from . import flash_decode
+        k, v, table, lens = self.get_layer_kv_cache(layer_idx)
+        ks, vs = self.layer_scales(layer_idx)
+        if ks is not None:
+            kwargs.setdefault("k_scale", ks)
+            kwargs.setdefault("v_scale", vs)
+        kwargs.setdefault("max_kv_len", max(self._host_len, 1))
+        return flash_decode(q, k, v, table, lens, sm_scale, **kwargs)
