@@ -67,8 +67,8 @@ def test_pack_unpack_layout():
     assert tda.pack_out_lse(out, lse, torch.float32).dtype == torch.float32
 
 
-def test_algorithmic_bytes_match_the_published_table():
-    # bytes per call of the uniform-length configurations
+def test_algorithmic_bytes_match_the_hand_computed_figures():
+    # bytes per call of the uniform-length configurations: KV + q + out + lse + table entries used + lengths (+ scales)
     assert wl.make_inputs("tiny").algorithmic_bytes() == 1_060_936
 
     def bytes_of(name):
