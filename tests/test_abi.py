@@ -153,9 +153,31 @@ def test_counters_of_the_work_queue_form():
     n = lib.fdk_counters_len(C.byref(a))
     assert n == 2
     assert lib.fdk_counters_len(None) == 0
-    # dry run ignores them; a real call would reject a short or misaligned array before launching anything
     a.counters, a.counters_len = 0x90000, n
     assert _decode_rc(a) == 0
+    # the work-queue form exists for forced split counts (chunk mode): there a short or misaligned array is refused,
+    # in a dry run as in a real call, before anything is launched
+    assert _decode_rc(_args(batch=4, num_splits=8, counters=0x90000, counters_len=n)) == 0
+    assert _decode_rc(_args(batch=4, num_splits=8, counters=0x90000, counters_len=1)) == _lib.FDK_EWORKSPACE
+    assert _decode_rc(_args(batch=4, num_splits=8, counters=0x90002, counters_len=n)) == _lib.FDK_EALIGN
+
+
+def test_dry_run_refuses_what_a_real_call_would_refuse():
+    lib = _lib.load()
+    # a block_table row addresses at most 2^30 tokens (32-bit token arithmetic in the kernels)
+    assert _decode_rc(_args(page_size=1 << 20, max_pages=1 << 10, table_stride_b=1 << 10,
+                            k_stride_page=(1 << 20) * 1024, v_stride_page=(1 << 20) * 1024)) == 0
+    rc = _decode_rc(_args(page_size=1 << 20, max_pages=(1 << 10) + 1, table_stride_b=(1 << 10) + 1,
+                          k_stride_page=(1 << 20) * 1024, v_stride_page=(1 << 20) * 1024))
+    assert rc == _lib.FDK_ESHAPE and b"2^30" in lib.fdk_last_error()
+    # more workgroups than a grid holds
+    big = dict(batch=1 << 22, num_splits=1024, workspace_bytes=1 << 62, q_stride_b=32 * 128, out_stride_b=32 * 128)
+    rc = _decode_rc(_args(**big))
+    assert rc == _lib.FDK_ESHAPE and b"grid" in lib.fdk_last_error()
+    a = _args(**big)
+    assert lib.fdk_decode_splitkv(C.byref(a), None) == _lib.FDK_ESHAPE
+    # a misaligned workspace
+    assert _decode_rc(_args(batch=4, workspace=0x80004)) == _lib.FDK_EALIGN
 
 
 def test_packed_output_needs_a_wider_row():
@@ -306,6 +328,7 @@ def test_kv_append_accepts_valid_arguments_and_rejects_bad_ones():
         ("q_out_stride_h", 127, _lib.FDK_ESHAPE),
         ("cs_stride_pos", 32, _lib.FDK_ESHAPE),
         ("table_stride_b", 255, _lib.FDK_ESHAPE),
+        ("new_tokens", 2 ** 31 - 1, _lib.FDK_ESHAPE),                 # batch * tokens * head rows beyond a grid
         ("k_stride_head", 64, _lib.FDK_ESHAPE),
         ("v_stride_tok", -8, _lib.FDK_ESHAPE),
         ("q_eps", float("nan"), _lib.FDK_ESHAPE),

@@ -61,6 +61,8 @@ constexpr int kChunkAlign = 64;     // split boundaries fall on multiples of 64 
 constexpr int kMinChunk = 64;       // shortest chunk (short contexts: latency matters more than the partials)
 constexpr int kMaxMinChunk = 512;   // long contexts are never split finer than this
 constexpr int kMaxSplits = 1024;
+constexpr int64_t kMaxTableTokens = (int64_t)1 << 30;
+constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and never asks the runtime
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
 
@@ -77,8 +79,10 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
     if (a->page_size <= 0) return fail(FDK_ESHAPE, "page_size %d <= 0", a->page_size);
     if (a->max_pages <= 0) return fail(FDK_ESHAPE, "max_pages %d <= 0", a->max_pages);
-    if ((int64_t)a->max_pages * a->page_size > INT32_MAX)
-        return fail(FDK_ESHAPE, "max_pages*page_size overflows int32");
+    // token positions, chunk bounds (start + chunk) and granule counts are 32-bit in the kernels
+    if ((int64_t)a->max_pages * a->page_size > kMaxTableTokens)
+        return fail(FDK_ESHAPE, "max_pages*page_size = %lld: a block_table row may address at most 2^30 tokens",
+                    (long long)((int64_t)a->max_pages * a->page_size));
     if (a->max_kv_len < 0) return fail(FDK_ESHAPE, "max_kv_len %d < 0", a->max_kv_len);
     if (a->num_splits < 0 || a->num_splits > kMaxSplits)
         return fail(FDK_ESHAPE, "num_splits %d outside [0, %d]", a->num_splits, kMaxSplits);
@@ -232,8 +236,9 @@ struct Resolved {
     fdk::CombineParams cp;
 };
 
-int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
-    int rc = make_plan(a, 0, &r->plan);
+int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) {
+    if (num_cus <= 0) num_cus = query_cus();
+    int rc = make_plan(a, num_cus, &r->plan);
     if (rc) return rc;
     const int S = r->plan.num_splits;
     const bool direct = direct_ok && S == 1;
@@ -260,7 +265,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, Resolved* r) {
     sp.part_o = part_o; sp.part_lse = part_lse;
     sp.out = a->out; sp.lse = a->lse;
     sp.counters = nullptr;
-    sp.num_cus = query_cus();
+    sp.num_cus = num_cus;
     sp.q_sb = a->q_stride_b; sp.q_sh = a->q_stride_h;
     sp.k_sp = a->k_stride_page; sp.k_st = a->k_stride_tok; sp.k_sh = a->k_stride_head;
     sp.v_sp = a->v_stride_page; sp.v_st = a->v_stride_tok; sp.v_sh = a->v_stride_head;
@@ -335,7 +340,7 @@ int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
     if (!plan) return fail(FDK_ENULL, "plan is null");
     int rc = validate(args, false, false);
     if (rc) return rc;
-    if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = 256;
+    if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = kDryRunCus;
     return make_plan(args, num_cus, plan);
 }
 
@@ -343,21 +348,11 @@ int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
     g_err[0] = 0;
     int rc = validate(args, true, false);
     if (rc) return rc;
-    if (args->flags & FDK_FLAG_DRY_RUN) {
-        fdk_plan_t plan;
-        rc = make_plan(args, 256, &plan);
-        if (rc) return rc;
-        if (plan.num_splits > 1 && args->batch > 0) {
-            const size_t need = fdk_workspace_bytes(args->batch, args->num_q_heads, args->head_dim, plan.num_splits);
-            if (!args->workspace) return fail(FDK_EWORKSPACE, "workspace is null; %zu bytes needed", need);
-            if (args->workspace_bytes < need)
-                return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed", args->workspace_bytes, need);
-        }
-        return FDK_OK;
-    }
     if (args->batch == 0) return FDK_OK;
+    // A dry run goes through everything the host decides (plan, workspace, counters) and stops before the launch.
+    const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
     Resolved r;
-    rc = resolve(args, true, &r);
+    rc = resolve(args, true, dry ? kDryRunCus : 0, &r);
     if (rc) return rc;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
     // work-queue form of the split kernel (matrix-core path only)
@@ -369,6 +364,7 @@ int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
                         (long long)fdk_counters_len(args));
         r.sp.counters = args->counters;
     }
+    if (dry) return FDK_OK;
     rc = launch_split(args, r, stream);
     if (rc) return rc;
     if (!r.sp.direct) {
@@ -382,10 +378,11 @@ int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {
     g_err[0] = 0;
     int rc = validate(args, false, true);
     if (rc) return rc;
-    if (args->batch == 0 || (args->flags & FDK_FLAG_DRY_RUN)) return FDK_OK;
+    if (args->batch == 0) return FDK_OK;
+    const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
     Resolved r;
-    rc = resolve(args, false, &r);
-    if (rc) return rc;
+    rc = resolve(args, false, dry ? kDryRunCus : 0, &r);
+    if (rc || dry) return rc;
     return launch_split(args, r, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
@@ -393,10 +390,11 @@ int fdk_combine(const fdk_decode_args* args, void* hip_stream) {
     g_err[0] = 0;
     int rc = validate(args, true, true);
     if (rc) return rc;
-    if (args->batch == 0 || (args->flags & FDK_FLAG_DRY_RUN)) return FDK_OK;
+    if (args->batch == 0) return FDK_OK;
+    const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
     Resolved r;
-    rc = resolve(args, false, &r);
-    if (rc) return rc;
+    rc = resolve(args, false, dry ? kDryRunCus : 0, &r);
+    if (rc || dry) return rc;
     rc = fdk::launch_combine(r.cp, reinterpret_cast<hipStream_t>(hip_stream));
     if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     return FDK_OK;
@@ -456,7 +454,8 @@ int fdk_kv_append(const fdk_kv_append_args* a, void* hip_stream) {
     if (!(a->q_eps == a->q_eps) || !(a->k_eps == a->k_eps) || a->q_eps < 0.f || a->k_eps < 0.f)
         return fail(FDK_ESHAPE, "eps must be non-negative numbers");
     if (a->batch == 0 || a->new_tokens == 0) return FDK_OK;
-    if ((int64_t)a->batch * a->new_tokens * (a->num_q_heads + 2 * a->num_kv_heads) > (int64_t)INT32_MAX * 4)
+    const int64_t head_rows = (int64_t)a->num_q_heads + 2 * (int64_t)a->num_kv_heads;
+    if ((int64_t)a->batch * a->new_tokens > (int64_t)INT32_MAX * 4 / head_rows)       // one wavefront per head row
         return fail(FDK_ESHAPE, "grid too large");
     if (!a->qkv || !a->k_weight || !a->cos || !a->sin || !a->block_table || !a->kv_lens || !a->k_cache || !a->v_cache)
         return fail(FDK_ENULL, "qkv / k_weight / cos / sin / block_table / kv_lens / k_cache / v_cache must be non-null");
