@@ -210,6 +210,10 @@ def test_plan_scales_splits_with_occupancy():
     p4 = _plan(_args(batch=4))
     assert p4.balanced == 0 and p4.num_splits > 1 and p4.chunk_tokens % 64 == 0
     assert p4.num_splits * p4.chunk_tokens >= 4096 > (p4.num_splits - 1) * p4.chunk_tokens
+    # chunk mode aims at one workgroup per compute unit and never launches more than there are compute units
+    assert p4.kv_heads_per_wg == 2 and p4.num_splits == 256 // (4 * 4)
+    p24 = _plan(_args(batch=24, max_pages=64, table_stride_b=64))       # 96 units, 1024 tokens
+    assert p24.balanced == 0 and p24.num_splits == 2 and p24.chunk_tokens == 512
     # few units, long context: balanced mode - two workgroups per compute unit share the KV ranges of the whole
     # batch, each gets a long share, and the workspace holds (shares + batch) slots per head block
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,

@@ -165,23 +165,23 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const int64_t units = (int64_t)batch * units_per_seq;
 
     // Split count: none when the (sequence, head block) units alone fill the compute units - a single pass
-    // then writes the final result and no combine runs.  Otherwise aim at two workgroups per compute unit.
+    // then writes the final result and no combine runs.  Otherwise the per-sequence chunks aim at one workgroup
+    // per compute unit and never more: on MI355X 256 workgroups finish 2-7 % sooner than 512 with the same
+    // total work, and a grid a little larger than what is resident at once runs in two rounds.
     // The shortest chunk grows with the context (max_len / 64, between kMinChunk and kMaxMinChunk tokens):
     // a short context is latency-bound and gains from every extra split, a long one pays for each partial
     // row it writes and re-reads.
     int64_t min_chunk = cdiv64(cdiv64(max_len, 64), kChunkAlign) * kChunkAlign;
     if (min_chunk < kMinChunk) min_chunk = kMinChunk;
     if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
-    int64_t splits;
+    const int64_t most_chunks = cdiv64(max_len, min_chunk);
+    const bool may_split = a->num_splits <= 0 && units < num_cus && most_chunks > 1;
+    int64_t splits = 1;
     if (a->num_splits > 0) {
         splits = a->num_splits;
-    } else if (units >= num_cus) {
-        splits = 1;
-    } else {
-        splits = cdiv64(2 * (int64_t)num_cus, units);
-        const int64_t cap = cdiv64(max_len, min_chunk);
-        if (splits > cap) splits = cap;
-        if (splits < 1) splits = 1;
+    } else if (may_split) {
+        splits = (int64_t)num_cus / units;
+        if (splits > most_chunks) splits = most_chunks;
     }
     memset(plan, 0, sizeof(*plan));
     plan->algo = algo;
@@ -192,7 +192,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // that a ragged batch loads every workgroup alike.  The workspace then holds (shares + batch) slots of
     // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
     const int64_t columns = (int64_t)batch * cdiv64(max_len, fdk::kBalanceGranule);   // granules of all sequences, at most
-    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && splits > 1 && batch <= kMaxBalancedBatch &&
+    if (algo == FDK_ALGO_MFMA && may_split && batch <= kMaxBalancedBatch &&
         columns < (1 << 30)) {                                            // the kernel counts granules in int32
         const int64_t gran = fdk::kBalanceGranule;
         int64_t shares = columns / (min_chunk / gran);
