@@ -194,7 +194,7 @@ def main():
         pools.append((mk(), mk()))
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
-                                max_kv_len=max(inp.kv_lens_host))
+                                max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
              for k, v in pools]
     plan = calls[0].plan
     alg_bytes = inp.algorithmic_bytes()
@@ -269,6 +269,7 @@ def main():
             "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "kv_pools_rotated": len(pools),
+            "host_length_hints": [min(inp.kv_lens_host), max(inp.kv_lens_host)],
         },
         "roofline": {
             "bound": "hbm",

@@ -224,6 +224,18 @@ def test_plan_scales_splits_with_occupancy():
     rows = (shares + 4) * units * p_long.kv_heads_per_wg * 8           # group = 8 heads per tile
     assert p_long.num_splits * 4 * 64 >= rows > (p_long.num_splits - 1) * 4 * 64
     assert shares * p_long.chunk_tokens >= 4 * 131072                   # the shares cover every sequence
+    # the same shape with a host-known lower bound close to the upper one: the batch is uniform, so per-sequence
+    # chunks (one workgroup per compute unit) replace the balanced shares; a looser bound changes nothing
+    long_kw = dict(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048, q_stride_b=64 * 128,
+                   out_stride_b=64 * 128, lse_stride_b=64)
+    p_uni = _plan(_args(min_kv_len=131072, **long_kw))
+    assert p_uni.balanced == 0 and p_uni.num_splits * (4 * 8 // p_uni.kv_heads_per_wg) == 256
+    assert p_uni.num_splits * p_uni.chunk_tokens == 131072
+    assert _plan(_args(min_kv_len=131072 * 31 // 32, **long_kw)).balanced == 0
+    assert _plan(_args(min_kv_len=131072 * 31 // 32 - 1, **long_kw)).balanced == 1
+    assert _decode_rc(_args(min_kv_len=-1)) == _lib.FDK_ESHAPE
+    assert _decode_rc(_args(max_kv_len=4096, min_kv_len=4097)) == _lib.FDK_ESHAPE
+    assert _decode_rc(_args(max_kv_len=4096, min_kv_len=4096)) == 0
     # a short context is latency-bound: chunk mode, split down to chunks of 64 tokens, never finer
     p_short = _plan(_args(batch=1, max_pages=8, table_stride_b=8))
     assert p_short.balanced == 0 and p_short.num_splits == 2 and p_short.chunk_tokens == 64

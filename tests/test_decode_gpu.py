@@ -365,6 +365,36 @@ def test_a_length_hint_that_is_too_small_loses_no_tokens(cuda_device, algo, kv_s
     _check(out, lse, q, k, v, table, lens, d ** -0.5, tag=f"small hint {algo} S={kv_split}")
 
 
+@pytest.mark.parametrize("true_lens", [[24000] * 4, [24000, 23990, 24000, 23900], [24000, 37, 1, 9000]])
+def test_the_lower_length_hint_selects_chunks_and_never_changes_results(cuda_device, true_lens):
+    # min_kv_len close to max_kv_len: per-sequence chunks instead of balanced shares.  The hint may be wrong (third
+    # case: the batch is ragged although the caller claims uniform lengths) - the result is the same, only slower.
+    g = torch.Generator().manual_seed(93)
+    hq, hkv, d, page = 32, 8, 128, 16
+    pages = [(24000 + page - 1) // page] * 4
+    pool = sum(pages)
+    q = torch.randn(4, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.randperm(pool, generator=g).to(torch.int32).view(4, pages[0]).to(cuda_device)
+    lens_t = _lens_t(true_lens, cuda_device)
+    args = (q, k, v, table, lens_t, d ** -0.5)
+    p_bal = tda.get_split_kv_plan(*args, max_kv_len=24000)
+    p_uni = tda.get_split_kv_plan(*args, max_kv_len=24000, min_kv_len=24000)
+    p_near = tda.get_split_kv_plan(*args, max_kv_len=24000, min_kv_len=23900)
+    p_far = tda.get_split_kv_plan(*args, max_kv_len=24000, min_kv_len=20000)
+    assert p_bal.balanced and p_far.balanced and not p_uni.balanced and not p_near.balanced
+    assert p_uni.num_splits == 256 // (4 * 8 // p_uni.kv_heads_per_wg)          # one workgroup per compute unit
+    out_b, lse_b = tda.flash_decode(*args, max_kv_len=24000)
+    out_u, lse_u = tda.flash_decode(*args, max_kv_len=24000, min_kv_len=24000)
+    torch.cuda.synchronize()
+    _check(out_u, lse_u, q, k, v, table, true_lens, d ** -0.5, tag=f"uniform hint {true_lens}")
+    torch.testing.assert_close(out_u.float(), out_b.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse_u, lse_b, atol=1e-4, rtol=1e-5)
+    with pytest.raises(ValueError, match="min_kv_len"):
+        tda.flash_decode(*args, max_kv_len=24000, min_kv_len=24001)
+
+
 def test_zero_length_sequence_is_defined(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=300), cuda_device)
     lens = _lens_t([300, 0, 17], cuda_device)

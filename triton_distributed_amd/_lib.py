@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 4
+FDK_ABI_VERSION = 5
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -44,7 +44,8 @@ class FdkDecodeArgs(C.Structure):
         ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
         ("block_table", C.c_void_p), ("table_stride_b", C.c_int64), ("kv_lens", C.c_void_p),
         ("batch", C.c_int32), ("num_q_heads", C.c_int32), ("num_kv_heads", C.c_int32), ("head_dim", C.c_int32),
-        ("page_size", C.c_int32), ("max_pages", C.c_int32), ("max_kv_len", C.c_int32), ("num_splits", C.c_int32),
+        ("page_size", C.c_int32), ("max_pages", C.c_int32), ("max_kv_len", C.c_int32),
+        ("min_kv_len", C.c_int32), ("num_splits", C.c_int32),
         ("sm_scale", C.c_float), ("soft_cap", C.c_float),
         ("out", C.c_void_p), ("out_stride_b", C.c_int64), ("out_stride_h", C.c_int64),
         ("out_dtype", C.c_int32), ("algo", C.c_int32),

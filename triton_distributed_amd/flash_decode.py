@@ -82,7 +82,7 @@ class SplitKvPlan:
 
 
 def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
-               k_scale, v_scale, algo, check_device=True) -> FdkDecodeArgs:
+               k_scale, v_scale, algo, check_device=True, min_kv_len=None) -> FdkDecodeArgs:
     if q.dim() != 3:
         raise ValueError(f"q must be [batch, q_heads, head_dim], got {tuple(q.shape)}")
     if k_cache.dim() != 4 or v_cache.dim() != 4:
@@ -136,6 +136,7 @@ def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv
     a.page_size = page_size
     a.max_pages = block_table.shape[1]
     a.max_kv_len = int(max_kv_len) if max_kv_len else 0
+    a.min_kv_len = int(min_kv_len) if min_kv_len else 0
     a.num_splits = int(kv_split) if kv_split and kv_split > 0 else 0
     a.sm_scale = float(sm_scale)
     a.soft_cap = float(soft_cap) if soft_cap else 0.0
@@ -152,10 +153,10 @@ def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
 
 
 def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, soft_cap=0.0, kv_split=-1,
-                      max_kv_len=None, algo="auto", num_cus: int = 0) -> SplitKvPlan:
+                      max_kv_len=None, algo="auto", num_cus: int = 0, min_kv_len=None) -> SplitKvPlan:
     """The split count / chunk length / algorithm a decode call with these tensors will use."""
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
-                   None, None, algo, check_device=False)
+                   None, None, algo, check_device=False, min_kv_len=min_kv_len)
     if num_cus > 0:
         a.flags |= _lib.FDK_FLAG_DRY_RUN
     return _plan_of(a, num_cus)
@@ -206,7 +207,7 @@ class PreparedDecode:
 def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
-                   work_queue=True) -> PreparedDecode:
+                   work_queue=True, min_kv_len=None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -217,7 +218,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
-                   k_scale, v_scale, algo)
+                   k_scale, v_scale, algo, min_kv_len=min_kv_len)
     batch, q_heads, d = q.shape
     plan = _plan_of(a)
     if packed_out is not None:
@@ -273,7 +274,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  kv_split: int = -1, max_kv_len: Optional[int] = None, k_scale: Optional[torch.Tensor] = None,
                  v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                  lse: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                 algo: str = "auto", stream=None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 algo: str = "auto", stream=None, min_kv_len: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Local (one GPU's share) split-KV GQA decode attention over a paged KV cache.
 
     q            [B, Hq, D] bf16/fp16, one query token per sequence
@@ -286,6 +287,8 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     kv_split     force this many KV splits (default: chosen from the shape and the CU count)
     max_kv_len   host-known upper bound of kv_lens, used only to size the splits
                  (default ``max_pages * P``)
+    min_kv_len   host-known lower bound of kv_lens (default: unknown).  A batch whose bounds lie within 1/32 of
+                 each other is cut into per-sequence chunks instead of balanced shares; results never depend on it
     k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
@@ -294,7 +297,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
         stream = _stream_handle(stream)               # looked up once: torch.cuda.current_stream() is not free
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
-                          out=out, lse=lse, workspace=workspace, algo=algo,
+                          out=out, lse=lse, workspace=workspace, algo=algo, min_kv_len=min_kv_len,
                           counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)

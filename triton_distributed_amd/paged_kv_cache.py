@@ -11,7 +11,8 @@ Differences, all additions:
   * ``dtype=torch.float8_e4m3fn`` keeps 1-byte pools plus per-layer, per-kv-head fp32 scales
     (``k_scale, v_scale [num_layers, Hkv]``, given by the caller);
   * the lengths are tracked on the host as well (``max_kv_len``), so the decode can be planned for the real
-    length without reading ``kv_lens`` back from the GPU - a hint that is too small never drops tokens;
+    length without reading ``kv_lens`` back from the GPU (both bounds: the sequences advance together, so
+    the decode may use per-sequence chunks) - a hint that is wrong never changes results;
   * ``append`` / ``decode`` run the two operators of this package on one layer's view.
 
 The class itself allocates with torch and launches nothing; it works on any torch device (the operators do not).
@@ -129,4 +130,5 @@ class PagedKVCache:
             kwargs.setdefault("k_scale", ks)
             kwargs.setdefault("v_scale", vs)
         kwargs.setdefault("max_kv_len", max(self._host_len, 1))
+        kwargs.setdefault("min_kv_len", self._host_len)          # all sequences advance together
         return flash_decode(q, k, v, table, lens, sm_scale, **kwargs)
