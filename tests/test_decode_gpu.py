@@ -942,12 +942,11 @@ def test_random_shapes_against_the_oracle(cuda_device, seed):
         ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
     scale_mult = float(rng.choice([0.5, 1.0, 1.0, 2.0]))
     scale = float(d ** -0.5) * scale_mult
-    if hint is not None and hint < max(lens):
-        hint_arg = hint                                # too small on purpose: costs balance, not tokens
-    else:
-        hint_arg = hint
+    # hints may be wrong in either direction (an upper bound below the longest sequence, a lower bound above the
+    # shortest): they cost balance, never tokens
+    low = None if rng.random() < 0.6 else int((hint if hint is not None else n_max) * rng.choice([0.25, 0.98, 1.0]))
     out, lse = tda.flash_decode(q, k, v, table, _lens_t(lens, cuda_device), scale, soft_cap=soft_cap, kv_split=kv_split,
-                                max_kv_len=hint_arg, k_scale=ks, v_scale=vs)
+                                max_kv_len=hint, min_kv_len=low, k_scale=ks, v_scale=vs)
     torch.cuda.synchronize()
     empty = [i for i, n in enumerate(lens) if n == 0]
     live = [i for i, n in enumerate(lens) if n > 0]
