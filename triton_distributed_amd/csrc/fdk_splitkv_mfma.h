@@ -201,8 +201,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const int n = min(tok0 + j * RPL + lrow, c_end - 1);      // clamp: always a valid, finite row
             const int slot = PM == PM_LANE_DIV ? n % p.page_size : (n & pmask);
             const int64_t pg = pi.pg[PM == PM_TILE ? 0 : j];
-            put(rg.k[j], *reinterpret_cast<const uint4*>(kbase + (pg * p.k_sp + (int64_t)slot * p.k_st) * ES));
-            put(rg.v[j], *reinterpret_cast<const uint4*>(vbase + (pg * p.v_sp + (int64_t)slot * p.v_st) * ES));
+            put(rg.k[j], load_stream16(kbase + (pg * p.k_sp + (int64_t)slot * p.k_st) * ES));
+            put(rg.v[j], load_stream16(vbase + (pg * p.v_sp + (int64_t)slot * p.v_st) * ES));
         }
     };
 
@@ -230,10 +230,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const char* vp = vplane + (pg * p.v_sp + (int64_t)slot0 * p.v_st) * ES;
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
-                put(rg.k[j], *reinterpret_cast<const uint4*>(kOffsetsInRegs ? kp + koff[j] : kp + j * kstep + koff[0]));
+                put(rg.k[j], load_stream16(kOffsetsInRegs ? kp + koff[j] : kp + j * kstep + koff[0]));
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
-                put(rg.v[j], *reinterpret_cast<const uint4*>(kOffsetsInRegs ? vp + voff[j] : vp + j * vstep + voff[0]));
+                put(rg.v[j], load_stream16(kOffsetsInRegs ? vp + voff[j] : vp + j * vstep + voff[0]));
         } else {
             issue(t, pi, rg);
         }
@@ -551,7 +551,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
             __syncthreads();
             item = s_next[0];
-            if (item >= p.total_items) break;
+            // unsigned: a queue head that was not zero on entry ends the queue instead of yielding a negative item
+            if ((unsigned)item >= (unsigned)p.total_items) break;
         }
     }
     if (threadIdx.x == 0) {                       // persistent chunk mode: leave the counters at zero

@@ -183,9 +183,9 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
         const char* vp[NJ];
         row_ptrs(T, pi, kp, vp);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) put(kt.k[j], *reinterpret_cast<const uint4*>(kp[j]));
+        for (int j = 0; j < NJ; ++j) put(kt.k[j], load_stream16(kp[j]));
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) put(kt.v[j], *reinterpret_cast<const uint4*>(vp[j]));
+        for (int j = 0; j < NJ; ++j) put(kt.v[j], load_stream16(vp[j]));
     };
     auto issue_masked = [&](int T, const PageIds& pi, KvTile& kt) {
         const char* kp[NJ];
@@ -196,8 +196,8 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
         for (int j = 0; j < NJ; ++j) {
             uint4 kk = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
             if (tok0 + j * ti_n * TPL + tok_in_tile0 < c_end) {
-                kk = *reinterpret_cast<const uint4*>(kp[j]);
-                vv = *reinterpret_cast<const uint4*>(vp[j]);
+                kk = load_stream16(kp[j]);
+                vv = load_stream16(vp[j]);
             }
             put(kt.k[j], kk);
             put(kt.v[j], vv);
