@@ -127,6 +127,12 @@ def test_valid_arguments_pass_dry_run():
     ("out_dtype", _lib.FDK_FP8_E4M3, _lib.FDK_EUNSUPPORTED),
     ("algo", 7, _lib.FDK_EUNSUPPORTED),
     ("sm_scale", float("nan"), _lib.FDK_ESHAPE),
+    ("sm_scale", float("inf"), _lib.FDK_ESHAPE),
+    ("sm_scale", float("-inf"), _lib.FDK_ESHAPE),
+    ("soft_cap", float("nan"), _lib.FDK_ESHAPE),
+    ("soft_cap", float("inf"), _lib.FDK_ESHAPE),
+    ("k_stride_tok", 1 << 27, _lib.FDK_ESHAPE),             # 16 rows of 2^28 bytes: offsets would not fit 32 bits
+    ("v_stride_tok", 1 << 27, _lib.FDK_ESHAPE),
 ])
 def test_bad_arguments_are_rejected_without_a_launch(field, value, code):
     rc = _decode_rc(_args(**{field: value}))
@@ -134,6 +140,13 @@ def test_bad_arguments_are_rejected_without_a_launch(field, value, code):
     assert len(_lib.load().fdk_last_error()) > 0
     with pytest.raises((ValueError, _lib.FdkError)):
         _lib.check(rc)
+
+
+def test_fp8_scale_pointers_must_be_aligned():
+    ok = dict(kv_dtype=_lib.FDK_FP8_E4M3, k_scale=0x90000, v_scale=0x90100)
+    assert _decode_rc(_args(**ok)) == 0
+    assert _decode_rc(_args(**{**ok, "k_scale": 0x90002})) == _lib.FDK_EALIGN
+    assert _decode_rc(_args(**{**ok, "v_scale": 0x90101})) == _lib.FDK_EALIGN
 
 
 def test_workspace_is_required_only_when_the_plan_splits():
@@ -273,6 +286,8 @@ def test_workspace_bytes_formula():
     assert lib.fdk_workspace_bytes(32, 32, 128, 4) % 256 == 0
     assert lib.fdk_workspace_bytes(0, 32, 128, 4) == 0
     assert lib.fdk_workspace_bytes(32, 32, 128, 0) == 0
+    # a product that does not fit size_t saturates instead of wrapping to a small number
+    assert lib.fdk_workspace_bytes(2**31 - 1, 2**31 - 1, 2**31 - 1, 2**31 - 1) == 2**64 - 1
 
 
 def test_combine_ranks_validation():
@@ -294,6 +309,20 @@ def test_combine_ranks_validation():
     a.num_ranks = 0
     assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
     assert lib.fdk_combine_ranks(None, None) == _lib.FDK_ENULL
+    # the merged-lse output: aligned fp32 rows of at least Hq elements
+    a.num_ranks, a.flags = 8, _lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE
+    a.lse, a.lse_stride_b_out = 0x4000, 32
+    assert lib.fdk_combine_ranks(C.byref(a), None) == 0
+    a.lse_stride_b_out = 31
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
+    a.lse, a.lse_stride_b_out = 0x4002, 32
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_EALIGN
+    # unpacked: the per-rank lse rows must hold Hq elements too
+    a.lse, a.flags, a.partial_lse = 0x4000, _lib.FDK_FLAG_DRY_RUN, 0x5000
+    a.lse_stride_r, a.lse_stride_b = 4 * 32, 16
+    assert lib.fdk_combine_ranks(C.byref(a), None) == _lib.FDK_ESHAPE
+    a.lse_stride_b = 32
+    assert lib.fdk_combine_ranks(C.byref(a), None) == 0
 
 
 def _append_args(**kw):

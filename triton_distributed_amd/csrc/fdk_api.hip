@@ -1,5 +1,7 @@
 // C ABI of the flash-decode kernels: argument validation, launch planning, dispatch.
 // Declarations and the reference interfaces they replace: include/fdk.h.
+#include <float.h>
+#include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -93,7 +95,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if (a->kv_dtype != a->q_dtype && a->kv_dtype != FDK_FP8_E4M3)
         return fail(FDK_EUNSUPPORTED, "kv_dtype %d must equal q_dtype or be fp8_e4m3", a->kv_dtype);
     if (a->algo < FDK_ALGO_AUTO || a->algo > FDK_ALGO_MFMA) return fail(FDK_EUNSUPPORTED, "algo %d", a->algo);
-    if (!(a->sm_scale == a->sm_scale)) return fail(FDK_ESHAPE, "sm_scale is NaN");
+    if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
+    if (!(a->soft_cap <= FLT_MAX)) return fail(FDK_ESHAPE, "soft_cap is not a finite number (<= 0 switches it off)");
     if (a->batch == 0) return FDK_OK;
 
     if (!a->q || !a->k_cache || !a->v_cache || !a->block_table || !a->kv_lens)
@@ -111,6 +114,12 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         if (ks[i] < 0) return fail(FDK_ESHAPE, "negative cache stride");
         if ((ks[i] * kes) % 16) return fail(FDK_EALIGN, "cache strides must be multiples of 16 bytes");
     }
+    // the kernels keep the byte offsets of a tile's 16 token rows relative to its first row in 32 bits
+    if (a->k_stride_tok * kes * 16 >= ((int64_t)1 << 32) || a->v_stride_tok * kes * 16 >= ((int64_t)1 << 32))
+        return fail(FDK_ESHAPE, "cache token stride too large: 16 rows must span less than 4 GiB");
+    if (a->kv_dtype == FDK_FP8_E4M3 &&
+        ((reinterpret_cast<uintptr_t>(a->k_scale) & 3u) || (reinterpret_cast<uintptr_t>(a->v_scale) & 3u)))
+        return fail(FDK_EALIGN, "k_scale / v_scale must be 4-byte aligned");
     if ((a->k_stride_head < a->head_dim || a->v_stride_head < a->head_dim) && a->num_kv_heads > 1)
         return fail(FDK_ESHAPE, "cache head stride < head_dim (k %lld, v %lld)", (long long)a->k_stride_head,
                     (long long)a->v_stride_head);
@@ -317,39 +326,8 @@ int launch_split(const fdk_decode_args* a, const Resolved& r, hipStream_t stream
     return FDK_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-int fdk_abi_version(void) { return FDK_ABI_VERSION; }
-
-const char* fdk_last_error(void) { return g_err; }
-
-int fdk_device_cus(void) { return query_cus(); }
-
-int64_t fdk_counters_len(const fdk_decode_args* a) {
-    if (!a || a->batch <= 0 || a->num_q_heads <= 0) return 0;
-    return 2;      // queue head, finished-workgroup count
-}
-
-size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim, int32_t num_splits) {
-    if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 0) return 0;
-    const size_t rows = (size_t)batch * (size_t)num_q_heads * (size_t)num_splits;
-    size_t bytes = rows * ((size_t)head_dim + 1) * sizeof(float);
-    return (bytes + 255) & ~(size_t)255;
-}
-
-int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
-    g_err[0] = 0;
-    if (!plan) return fail(FDK_ENULL, "plan is null");
-    int rc = validate(args, false, false);
-    if (rc) return rc;
-    if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = kDryRunCus;
-    return make_plan(args, num_cus, plan);
-}
-
-int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
-    g_err[0] = 0;
+// Split launch + combine launch (a single launch for a one-split plan); the body of fdk_decode and fdk_decode_static.
+int decode_impl(const fdk_decode_args* args, void* hip_stream) {
     int rc = validate(args, true, false);
     if (rc) return rc;
     if (args->batch == 0) return FDK_OK;
@@ -376,6 +354,44 @@ int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
         if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
     return FDK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fdk_abi_version(void) { return FDK_ABI_VERSION; }
+
+const char* fdk_last_error(void) { return g_err; }
+
+int fdk_device_cus(void) { return query_cus(); }
+
+int64_t fdk_counters_len(const fdk_decode_args* a) {
+    if (!a || a->batch <= 0 || a->num_q_heads <= 0) return 0;
+    return 2;      // queue head, finished-workgroup count
+}
+
+size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim, int32_t num_splits) {
+    if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 0) return 0;
+    // batch * heads * splits < 2^93 would overflow: saturate instead, so that no buffer ever passes the size check
+    const unsigned __int128 rows = (unsigned __int128)batch * (unsigned __int128)num_q_heads * (unsigned __int128)num_splits;
+    const unsigned __int128 bytes = rows * ((unsigned __int128)head_dim + 1) * sizeof(float) + 255;
+    if (bytes > (unsigned __int128)SIZE_MAX) return SIZE_MAX;
+    return (size_t)bytes & ~(size_t)255;
+}
+
+int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
+    g_err[0] = 0;
+    if (!plan) return fail(FDK_ENULL, "plan is null");
+    int rc = validate(args, false, false);
+    if (rc) return rc;
+    if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = kDryRunCus;
+    return make_plan(args, num_cus, plan);
+}
+
+int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
+    g_err[0] = 0;
+    return decode_impl(args, hip_stream);
 }
 
 int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {
@@ -421,6 +437,11 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
     if (!packed && !a->partial_lse) return fail(FDK_ENULL, "partial_lse is null and FDK_FLAG_PACK_LSE is not set");
     if (a->stride_h < a->head_dim + (packed ? 1 : 0)) return fail(FDK_ESHAPE, "stride_h too small");
     if (a->out_stride_h < a->head_dim) return fail(FDK_ESHAPE, "out_stride_h too small");
+    if (a->lse && (reinterpret_cast<uintptr_t>(a->lse) & 3u)) return fail(FDK_EALIGN, "lse not 4-byte aligned");
+    if (a->lse && a->lse_stride_b_out < a->num_q_heads)
+        return fail(FDK_ESHAPE, "lse_stride_b_out %lld < Hq %d", (long long)a->lse_stride_b_out, a->num_q_heads);
+    if (!packed && a->lse_stride_b < a->num_q_heads)
+        return fail(FDK_ESHAPE, "lse_stride_b %lld < Hq %d", (long long)a->lse_stride_b, a->num_q_heads);
     if (a->flags & FDK_FLAG_DRY_RUN) return FDK_OK;
     fdk::CombineRanksParams p;
     memset(&p, 0, sizeof(p));

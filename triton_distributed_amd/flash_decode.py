@@ -163,19 +163,45 @@ def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, s
 
 
 _COUNTER_CACHE = {}
+_SCRATCH_CACHE = {}
 
 
-def _stream_counters(device: torch.device, stream, n: int = 64) -> torch.Tensor:
-    """Zeroed int32 counters shared by the calls issued on one stream (they run in order, and every call
-    leaves the counters zero), so the convenience entry points need no fill launch per call."""
-    if device.type != "cuda":
-        return None                                   # the caller is about to be told that there is no CPU path
+def _capturing() -> bool:
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
+def _stream_counters(device: torch.device, stream, n: int = 64) -> Optional[torch.Tensor]:
+    """Zeroed int32 counters shared by the eager calls issued on one stream (they run in order, and every call
+    leaves the counters zero), so the convenience entry points need no fill launch per call.  A call made while
+    its stream is capturing a HIP graph gets counters of its own instead (None here: ``prepare_decode`` then
+    allocates them): a replay may run on another stream and overlap eager calls on this one."""
+    if device.type != "cuda" or _capturing():
+        return None                                   # CPU tensors: the caller is about to be told there is no CPU path
     key = (device.index, _stream_handle(stream))
     t = _COUNTER_CACHE.get(key)
     if t is None or t.numel() < n:
         t = torch.zeros(n, dtype=torch.int32, device=device)
         _COUNTER_CACHE[key] = t
     return t
+
+
+def _stream_scratch(device: torch.device, stream, nbytes: int) -> Optional[torch.Tensor]:
+    """fp32 scratch for the split partials of the convenience entry points, kept per (device, stream) and grown on
+    demand: calls on one stream run in order, so they can share it.  Not used while capturing (see above)."""
+    if device.type != "cuda" or nbytes <= 0 or _capturing():
+        return None
+    key = (device.index, _stream_handle(stream))
+    t = _SCRATCH_CACHE.get(key)
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _SCRATCH_CACHE[key] = t
+    return t
+
+
+def _forget_stream_state(device: torch.device, stream) -> None:
+    """After a launch that failed the shared counters may not be zero any more: never hand them out again."""
+    if device.type == "cuda":
+        _COUNTER_CACHE.pop((device.index, _stream_handle(stream)), None)
 
 
 class PreparedDecode:
@@ -193,7 +219,10 @@ class PreparedDecode:
         self._ref = C.byref(args)
 
     def run(self, stream=None):
-        _lib.check(_LIB.fdk_decode(self._ref, _stream_handle(stream)))
+        rc = _LIB.fdk_decode(self._ref, _stream_handle(stream))
+        if rc > 0:                                    # a launch failed (rejected arguments launch nothing)
+            _forget_stream_state(self.out.device, stream)
+        _lib.check(rc)
         return self.out, self.lse
 
     def run_splitkv(self, stream=None):
@@ -207,14 +236,16 @@ class PreparedDecode:
 def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
-                   work_queue=True, min_kv_len=None) -> PreparedDecode:
+                   work_queue=True, min_kv_len=None, stream_scratch=None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
     dtype) in ``[..., D]`` - the reference's ``output_combine`` layout - instead of ``out``.
     ``counters``: zeroed int32 tensor for the work-queue form of a split decode (a fixed set of workgroups pulls
     the work items, which keeps ragged batches balanced); by default the call owns a private one.
-    ``work_queue=False`` launches one workgroup per item instead."""
+    ``work_queue=False`` launches one workgroup per item instead.
+    ``stream_scratch``: a stream (handle); scratch that the call has to provide itself is then taken from a buffer
+    kept per (device, stream) instead of a fresh allocation - only for calls that are issued on that stream at once."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -250,6 +281,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                                       workspace.numel() * workspace.element_size() < need or
                                       workspace.data_ptr() % 16):
             workspace = None        # too small / unusable: take our own
+        if workspace is None and stream_scratch is not None:
+            workspace = _stream_scratch(q.device, stream_scratch, need)      # shared by the calls of one stream
         if workspace is None:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         a.workspace = workspace.data_ptr()
@@ -298,6 +331,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
                           out=out, lse=lse, workspace=workspace, algo=algo, min_kv_len=min_kv_len,
+                          stream_scratch=stream if q.is_cuda else None,
                           counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)
@@ -317,7 +351,8 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
-                          want_lse=False, counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None,
+                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     call.run(stream)
     return output_combine
@@ -330,7 +365,8 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
-                          want_lse=False, counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None,
+                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)[0]
 
@@ -356,16 +392,16 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
     The reference runs a fixed grid of 132 programs that loop over (sequence, head, split) items and merge after a
     grid barrier on the int32 ``workspace``.  Here the same split count (32 unless ``kv_split`` says otherwise) runs
     as the work-queue form of the split kernel - two workgroups per compute unit pulling items - followed by the
-    combine kernel.  ``workspace`` is used as the queue's counters when it is a zeroed int32 GPU tensor with at
-    least two elements (the kernel leaves it zero); otherwise per-stream counters of this module are used.  The
-    result is in q's dtype (the reference allocates float16 whatever q is)."""
+    combine kernel.  ``workspace`` is ignored: the reference's barrier works with any initial contents of it
+    (common_ops.py:57-81), whereas the queue's counters must be zero on entry, so the library always uses counters
+    of its own (per stream, left at zero by every call).  The result is in q's dtype (the reference allocates
+    float16 whatever q is)."""
     splits = 32 if kv_split == -1 else kv_split
     if q.is_cuda:
         stream = _stream_handle(stream)
-    ctr = workspace if (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.dtype == torch.int32 and
-                        workspace.numel() >= 2 and workspace.is_contiguous()) else _stream_counters(q.device, stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap, kv_split=splits,
-                          workspace=_as_scratch(output_split), out=output_combine, want_lse=False, counters=ctr)
+                          workspace=_as_scratch(output_split), out=output_combine, want_lse=False,
+                          stream_scratch=stream if q.is_cuda else None, counters=_stream_counters(q.device, stream))
     return call.run(stream)[0]
 
 
@@ -420,6 +456,9 @@ def inter_rank_combine(all_ranks_output: torch.Tensor, global_kv_lens: torch.Ten
         raise ValueError("inputs must live on the GPU; there is no CPU path")
     if final_output is None:
         final_output = torch.empty((batch, q_heads, d), dtype=all_ranks_output.dtype, device=all_ranks_output.device)
+    elif tuple(final_output.shape) != (batch, q_heads, d) or final_output.stride(-1) != 1 or \
+            final_output.device != all_ranks_output.device:
+        raise ValueError(f"final_output must be a GPU tensor [B, Hq, D] = {(batch, q_heads, d)} with contiguous D")
     a = FdkCombineRanksArgs()
     a.struct_size = C.sizeof(FdkCombineRanksArgs)
     a.flags = _lib.FDK_FLAG_PACK_LSE if packed else 0
@@ -438,8 +477,11 @@ def inter_rank_combine(all_ranks_output: torch.Tensor, global_kv_lens: torch.Ten
     a.out = final_output.data_ptr()
     a.out_stride_b, a.out_stride_h = final_output.stride(0), final_output.stride(1)
     if lse_out is not None:
+        if lse_out.dtype != torch.float32 or tuple(lse_out.shape) != (batch, q_heads) or lse_out.stride(-1) != 1 or \
+                lse_out.device != all_ranks_output.device:
+            raise ValueError(f"lse_out must be an fp32 GPU tensor [B, Hq] = {(batch, q_heads)} with contiguous heads")
         a.lse = lse_out.data_ptr()
-        a.lse_stride_b_out = lse_out.stride(0)
+        a.lse_stride_b_out = lse_out.stride(0) if batch > 1 else max(lse_out.stride(0), q_heads)
     _lib.check(_LIB.fdk_combine_ranks(C.byref(a), _stream_handle(stream)))
     return final_output
 
