@@ -149,6 +149,23 @@ def test_fp8_scale_pointers_must_be_aligned():
     assert _decode_rc(_args(**{**ok, "v_scale": 0x90101})) == _lib.FDK_EALIGN
 
 
+def test_static_scratch_entry_validates_like_fdk_decode():
+    lib = _lib.load()
+    # needs neither workspace nor counters, whatever the plan
+    assert lib.fdk_decode_static(C.byref(_args(workspace=None, workspace_bytes=0)), None) == 0
+    assert lib.fdk_decode_static(C.byref(_args(batch=4, workspace=None, workspace_bytes=0)), None) == 0, lib.fdk_last_error()
+    assert lib.fdk_decode_static(C.byref(_args(num_splits=8, workspace=None, workspace_bytes=0)), None) == 0
+    # partials beyond the static scratch: 512 sequences x 32 heads x 64 splits x 129 fp32 = 541 MB
+    big = _args(batch=512, num_splits=64, workspace=None, workspace_bytes=0)
+    assert lib.fdk_workspace_bytes(512, 32, 128, 64) > _lib.FDK_STATIC_SCRATCH_BYTES
+    assert lib.fdk_decode_static(C.byref(big), None) == _lib.FDK_EWORKSPACE
+    assert b"static scratch" in lib.fdk_last_error()
+    # and the usual rejections
+    assert lib.fdk_decode_static(None, None) == _lib.FDK_ENULL
+    assert lib.fdk_decode_static(C.byref(_args(out=None)), None) == _lib.FDK_ENULL
+    assert lib.fdk_decode_static(C.byref(_args(head_dim=96)), None) == _lib.FDK_EUNSUPPORTED
+
+
 def test_workspace_is_required_only_when_the_plan_splits():
     # 32 sequences x 8 kv heads fill 256 compute units on their own: one pass, no scratch
     assert _decode_rc(_args(workspace=None, workspace_bytes=0)) == 0

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 5
+FDK_ABI_VERSION = 6
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -21,10 +21,12 @@ FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK
 FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
 # flags
 FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN = 1, 2
+FDK_STATIC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (
     "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
     "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len", "fdk_kv_append",
+    "fdk_decode_static",
 )
 
 
@@ -123,7 +125,7 @@ def load() -> C.CDLL:
     lib.fdk_plan.argtypes = [C.POINTER(FdkDecodeArgs), C.c_int, C.POINTER(FdkPlan)]
     lib.fdk_workspace_bytes.restype = C.c_size_t
     lib.fdk_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32]
-    for name in ("fdk_decode", "fdk_decode_splitkv", "fdk_combine"):
+    for name in ("fdk_decode", "fdk_decode_static", "fdk_decode_splitkv", "fdk_combine"):
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.POINTER(FdkDecodeArgs), C.c_void_p]

@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "fdk_device.h"
 
 namespace {
@@ -67,6 +69,33 @@ constexpr int64_t kMaxTableTokens = (int64_t)1 << 30;
 constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and never asks the runtime
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
+
+// Scratch of fdk_decode_static: one copy per GPU, part of the loaded code object, never allocated or freed.
+constexpr size_t kStaticScratchBytes = FDK_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};      // device address of g_static_scratch on each GPU
+
+// Device address of the static scratch on the current device, resolved once per device.
+int static_scratch_of_current_device(void** ptr) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail((int)e, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(FDK_EUNSUPPORTED, "device index %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess || !sym)
+            return fail(e != hipSuccess ? (int)e : FDK_EWORKSPACE, "hipGetSymbolAddress(static scratch) failed on device %d: %s",
+                        dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = sym;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return FDK_OK;
+}
 
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
     if (!a) return fail(FDK_ENULL, "args is null");
@@ -392,6 +421,37 @@ int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
 int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
     g_err[0] = 0;
     return decode_impl(args, hip_stream);
+}
+
+int fdk_decode_static(const fdk_decode_args* args, void* hip_stream) {
+    g_err[0] = 0;
+    int rc = validate(args, true, false);
+    if (rc) return rc;
+    if (args->batch == 0) return FDK_OK;
+    const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
+    fdk_plan_t plan;
+    rc = make_plan(args, dry ? kDryRunCus : 0, &plan);
+    if (rc) return rc;
+    fdk_decode_args a = *args;
+    a.workspace = nullptr;
+    a.workspace_bytes = 0;
+    a.counters = nullptr;          // one workgroup per item: nothing in the scratch has to start at zero
+    a.counters_len = 0;
+    if (plan.num_splits > 1) {
+        const size_t need = fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits);
+        if (need > kStaticScratchBytes)
+            return fail(FDK_EWORKSPACE,
+                        "fdk_decode_static: the partials of %d splits need %zu bytes, the static scratch holds %zu; "
+                        "use fdk_decode with a caller-owned workspace", plan.num_splits, need, kStaticScratchBytes);
+        if (dry) {
+            a.workspace = reinterpret_cast<void*>(uintptr_t(256));      // never dereferenced in a dry run
+        } else {
+            rc = static_scratch_of_current_device(&a.workspace);
+            if (rc) return rc;
+        }
+        a.workspace_bytes = kStaticScratchBytes;
+    }
+    return decode_impl(&a, hip_stream);
 }
 
 int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {

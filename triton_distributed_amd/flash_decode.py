@@ -225,6 +225,12 @@ class PreparedDecode:
         _lib.check(rc)
         return self.out, self.lse
 
+    def run_static(self, stream=None):
+        """The same call with the split partials in the library's static scratch (``fdk_decode_static``): no
+        workspace, no allocation of any kind.  Calls that overlap in time on one GPU race on that scratch."""
+        _lib.check(_LIB.fdk_decode_static(self._ref, _stream_handle(stream)))
+        return self.out, self.lse
+
     def run_splitkv(self, stream=None):
         _lib.check(_LIB.fdk_decode_splitkv(self._ref, _stream_handle(stream)))
 
@@ -236,7 +242,7 @@ class PreparedDecode:
 def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
-                   work_queue=True, min_kv_len=None, stream_scratch=None) -> PreparedDecode:
+                   work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -245,7 +251,9 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     the work items, which keeps ragged batches balanced); by default the call owns a private one.
     ``work_queue=False`` launches one workgroup per item instead.
     ``stream_scratch``: a stream (handle); scratch that the call has to provide itself is then taken from a buffer
-    kept per (device, stream) instead of a fresh allocation - only for calls that are issued on that stream at once."""
+    kept per (device, stream) instead of a fresh allocation - only for calls that are issued on that stream at once.
+    ``static_scratch=True`` binds no workspace and no counters: the call is then to be issued with
+    ``run_static()``, which keeps the split partials in the library's own static scratch."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -276,6 +284,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         a.lse = lse.data_ptr()
         a.lse_stride_b = lse.stride(0) if batch > 1 else max(lse.stride(0), q_heads)
     need = plan.workspace_bytes if (plan.num_splits > 1 or always_workspace) else 0
+    if static_scratch:
+        need, work_queue, workspace = 0, False, None
     if need:
         if workspace is not None and (not workspace.is_cuda or not workspace.is_contiguous() or
                                       workspace.numel() * workspace.element_size() < need or
