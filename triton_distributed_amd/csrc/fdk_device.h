@@ -236,6 +236,27 @@ __device__ __forceinline__ void store_out(void* base, int64_t idx, float x, int 
     }
 }
 
+// Store four consecutive output elements; one vector store when the address allows it.
+__device__ __forceinline__ void store_out4(void* base, int64_t idx, float4 x, int dtype) {
+    if (dtype == FDK_FP32) {
+        float* q = reinterpret_cast<float*>(base) + idx;
+        if ((reinterpret_cast<uintptr_t>(q) & 15u) == 0) {
+            *reinterpret_cast<float4*>(q) = x;
+        } else {
+            q[0] = x.x; q[1] = x.y; q[2] = x.z; q[3] = x.w;
+        }
+        return;
+    }
+    uint16_t* q = reinterpret_cast<uint16_t*>(base) + idx;
+    const uint2 v = dtype == FDK_BF16 ? make_uint2(Pack2<FDK_BF16>::pack(x.x, x.y), Pack2<FDK_BF16>::pack(x.z, x.w))
+                                      : make_uint2(Pack2<FDK_FP16>::pack(x.x, x.y), Pack2<FDK_FP16>::pack(x.z, x.w));
+    if ((reinterpret_cast<uintptr_t>(q) & 7u) == 0) {
+        *reinterpret_cast<uint2*>(q) = v;
+    } else {
+        q[0] = (uint16_t)v.x; q[1] = (uint16_t)(v.x >> 16); q[2] = (uint16_t)v.y; q[3] = (uint16_t)(v.y >> 16);
+    }
+}
+
 #endif  // __HIPCC__
 
 }  // namespace fdk

@@ -393,45 +393,78 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     }
 
     // ---- merge: lane groups (sum of l), then the wavefronts that share a kv head through LDS --------------
+    // A wave leaves its accumulators in its own scratch as [column block][lane] float4, i.e. exactly as its lanes
+    // hold them: every LDS instruction then touches one contiguous kilobyte.  The waves of a head share the
+    // column blocks; lane (h = c, a) of the merging wave reads the same lane slot of every wave's scratch and
+    // owns output columns 16 db + 4 a .. + 3 of head h.  Lanes of the padding heads neither write nor read.
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
-    float* my_o = reinterpret_cast<float*>(my_lds);          // [16 heads][D] fp32 = this wave's scratch
+    const bool live = c < heads_here;
+    float4* my_o = reinterpret_cast<float4*>(my_lds);
+    if (live) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-        *reinterpret_cast<float4*>(my_o + c * D + 16 * db + 4 * a) =
-            make_float4(acc[db].x, acc[db].y, acc[db].z, acc[db].w);
-    if (a == 0) {
-        sm_m[wave * 16 + c] = m_run;
-        sm_l[wave * 16 + c] = l_run;
+        for (int db = 0; db < DB; ++db) my_o[db * 64 + lane] = make_float4(acc[db].x, acc[db].y, acc[db].z, acc[db].w);
+        if (a == 0) {
+            sm_m[wave * 16 + c] = m_run;
+            sm_l[wave * 16 + c] = l_run;
+        }
     }
     if (ti_n > 1) __syncthreads();                           // ti_n == 1: a wave reads back only its own rows
-    const float* all_o = reinterpret_cast<const float*>(lds);
-    // wave w writes the rows of kv head (w % nh), sharing the work with the waves of the same head
-    for (int idx = tix * 64 + lane; idx < heads_here * D; idx += ti_n * 64) {
-        const int g = idx / D, d = idx % D;
+    if (live) {
+        constexpr int kMaxShare = 4;                         // at most four wavefronts share a kv head
+        float mw[kMaxShare], lw[kMaxShare];
         float mx = -INFINITY;
-        for (int t = 0; t < ti_n; ++t) mx = fmaxf(mx, sm_m[(hl + nh * t) * 16 + g]);
-        float o = 0.f, l = 0.f;
-        for (int t = 0; t < ti_n; ++t) {
-            const int w = hl + nh * t;
-            const float sc = fast_exp2(sm_m[w * 16 + g] - mx);     // mx is finite: the chunk holds >= 1 token
-            o += all_o[w * (kScratch / 4) + g * D + d] * sc;
-            l += sm_l[w * 16 + g] * sc;
-        }
-        const float res = o * vscale / l;
-        const int hq = head0 + g;
-        const float lse_nat = (mx + fast_log2(l)) * kLn2;
-        if (p.direct) {
-            const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh;
-            store_out(p.out, ob + d, res, p.out_dtype);
-            if (d == 0) {
-                if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
-                if (p.pack_lse) store_out(p.out, ob + D, lse_nat, p.out_dtype);
+#pragma unroll
+        for (int t = 0; t < kMaxShare; ++t) {
+            mw[t] = -INFINITY;
+            lw[t] = 0.f;
+            if (t < ti_n) {
+                mw[t] = sm_m[(hl + nh * t) * 16 + c];
+                lw[t] = sm_l[(hl + nh * t) * 16 + c];
             }
-        } else {
-            const int64_t row = prow0 + (int64_t)g * prow_step;
-            p.part_o[row * D + d] = res;
-            if (d == 0) p.part_lse[row] = lse_nat;
+            mx = fmaxf(mx, mw[t]);
+        }
+        float sc[kMaxShare], l = 0.f;
+#pragma unroll
+        for (int t = 0; t < kMaxShare; ++t) {
+            sc[t] = fast_exp2(mw[t] - mx);                   // mx is finite: the chunk holds >= 1 token
+            l += lw[t] * sc[t];
+        }
+        const float norm = vscale * fast_rcp(l);
+        const int hq = head0 + c;
+        const float lse_nat = (mx + fast_log2(l)) * kLn2;
+        for (int db = tix; db < DB; db += ti_n) {
+            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int t = 0; t < kMaxShare; ++t) {
+                if (t < ti_n) {
+                    const float4 x = reinterpret_cast<const float4*>(lds + (hl + nh * t) * kScratch)[db * 64 + lane];
+                    o.x += x.x * sc[t];
+                    o.y += x.y * sc[t];
+                    o.z += x.z * sc[t];
+                    o.w += x.w * sc[t];
+                }
+            }
+            o.x *= norm;
+            o.y *= norm;
+            o.z *= norm;
+            o.w *= norm;
+            const int d0 = 16 * db + 4 * a;
+            if (p.direct) {
+                const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0;
+                store_out4(p.out, ob, o, p.out_dtype);
+            } else {
+                const int64_t row = prow0 + (int64_t)c * prow_step;
+                *reinterpret_cast<float4*>(p.part_o + row * D + d0) = o;
+            }
+        }
+        if (tix == 0 && a == 0) {
+            if (p.direct) {
+                if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
+                if (p.pack_lse) store_out(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + D, lse_nat, p.out_dtype);
+            } else {
+                p.part_lse[prow0 + (int64_t)c * prow_step] = lse_nat;
+            }
         }
     }
 
