@@ -35,17 +35,21 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--config", default="llama3_8b_b32")
     ap.add_argument("--rotate", type=int, default=2,
-                    help="distinct KV pools cycled through, so the working set exceeds the 256 MB memory-side cache")
+                    help="distinct KV pools cycled through, so the working set exceeds the 256 MB memory-side cache "
+                         "(raised automatically until the pools together exceed 1 GB)")
     ap.add_argument("--kv-split", type=int, default=-1)
     ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
-    ap.add_argument("--op", default="decode", choices=["decode", "kv_append"],
+    ap.add_argument("--op", default="decode", choices=["decode", "kv_append", "ceiling"],
                     help="decode: the hot path (default); kv_append: the step before it (RMSNorm + rotary + "
-                         "paged append of one new token per sequence) at the same shape")
+                         "paged append of one new token per sequence) at the same shape; ceiling: what the memory "
+                         "system delivers for this configuration with no arithmetic in the way (a streaming read "
+                         "of as many bytes, and the split kernel reduced to its load pipeline) next to the kernel")
     return ap.parse_args()
 
 
@@ -96,7 +100,7 @@ def cpu_baseline(inp, budget_s: float):
         "us_per_call": est_call_s * 1e6,
         "cores": cores,
         "kind": "port",
-        "sample": (f"oracle ref_paged_attn (torch CPU, bf16) on sequences 0..{n_rows - 1} of {batch}, best of 3, "
+        "sample": (f"oracle ref_paged_attn (torch CPU, {inp.cfg.q_dtype}) on sequences 0..{n_rows - 1} of {batch}, best of 3, "
                    f"scaled by attended tokens ({tokens_sample}/{tokens_all})" +
                    ("" if n_rows < batch else "; full batch")),
     }
@@ -160,6 +164,85 @@ def bench_kv_append(args):
     }), flush=True)
 
 
+def _time_launches(torch, fn, n_iter, warm=10):
+    """Average microseconds per call of fn(i), HIP events on the current stream around n_iter back-to-back calls."""
+    for i in range(warm):
+        fn(i)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(n_iter):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n_iter
+
+
+def bench_ceiling(args):
+    """Load-only figures for one configuration, each timed like the kernel itself (events around back-to-back
+    launches that cycle through two KV pools):
+      linear_read      a streaming read of as many bytes as the call attends to, with and without the non-temporal hint
+      load_pipeline    the split kernel's own pieces, addresses and load instructions without the arithmetic
+      kernel           the split kernel"""
+    import torch
+    import triton_distributed_amd as tda
+    from triton_distributed_amd import workloads as wl
+
+    dev = torch.device("cuda:0")
+    inp = wl.make_inputs(args.config).to(dev)
+    if inp.cfg.kv_dtype == "fp8_e4m3" or inp.cfg.head_dim != 128:
+        print("--op ceiling: the load-pipeline probe is built for head_dim 128 and a 16-bit cache", file=sys.stderr)
+        sys.exit(2)
+    alg_bytes = inp.algorithmic_bytes()
+    g = torch.Generator(device=dev).manual_seed(inp.cfg.seed + 100)
+    pools = [(inp.k_cache, inp.v_cache),
+             tuple(torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype) for _ in range(2))]
+    kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
+              max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+    real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
+    probe = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, probe_loads=True, **kw)
+             for k, v in pools]
+    plan = real[0].plan
+    single_pass = plan.num_splits == 1
+    n_iter = args.steps
+    kv_bytes = sum(inp.kv_lens_host) * inp.cfg.kv_heads * 2 * inp.cfg.head_dim * 2
+    lin_bytes = max(kv_bytes // 2 // 65536 * 65536, 1 << 20)       # per buffer: the K half, then the V half
+    lin = [torch.randint(0, 255, (lin_bytes,), dtype=torch.uint8, device=dev) for _ in range(4)]
+
+    def linear(nt):
+        # one "call" = two launches (K-sized and V-sized buffer), four buffers in rotation
+        def fn(i):
+            tda.probe_linear_read(lin[(2 * i) % 4], nontemporal=nt)
+            tda.probe_linear_read(lin[(2 * i + 1) % 4], nontemporal=nt)
+        return fn
+
+    res = {}
+    res["linear_read_nt_us"] = _time_launches(torch, linear(True), n_iter)
+    res["linear_read_plain_us"] = _time_launches(torch, linear(False), n_iter)
+    res["load_pipeline_us"] = _time_launches(torch, lambda i: probe[i % 2].run(), n_iter)
+    res["kernel_us"] = _time_launches(torch, (lambda i: real[i % 2].run()) if single_pass else
+                                      (lambda i: real[i % 2].run_splitkv()), n_iter)
+    gb = lambda us, nbytes: round(nbytes / us / 1e3, 1)
+    print(json.dumps({
+        "metric": f"load-only ceilings of the decode path, {args.config}", "unit": "us per launch (GB/s, % of 8 TB/s)",
+        "config": {"workload": f"{args.config}: {inp.cfg.description}", "algorithmic_bytes_per_call": alg_bytes,
+                   "num_splits": plan.num_splits, "balanced": plan.balanced, "workgroups": plan.workgroups,
+                   "kv_heads_per_wg": plan.kv_heads_per_wg, "forced_kv_split": args.kv_split if args.kv_split > 0 else None},
+        "linear_read_bytes": 2 * lin_bytes,
+        "linear_read_nontemporal": {"us": round(res["linear_read_nt_us"], 2), "GBps": gb(res["linear_read_nt_us"], 2 * lin_bytes),
+                                    "pct_of_peak": round(gb(res["linear_read_nt_us"], 2 * lin_bytes) / 80, 2),
+                                    "note": "two launches of 512 workgroups per figure"},
+        "linear_read_plain": {"us": round(res["linear_read_plain_us"], 2), "GBps": gb(res["linear_read_plain_us"], 2 * lin_bytes),
+                              "pct_of_peak": round(gb(res["linear_read_plain_us"], 2 * lin_bytes) / 80, 2)},
+        "load_pipeline_only": {"us": round(res["load_pipeline_us"], 2), "GBps": gb(res["load_pipeline_us"], alg_bytes),
+                               "pct_of_peak": round(gb(res["load_pipeline_us"], alg_bytes) / 80, 2)},
+        "split_kernel": {"us": round(res["kernel_us"], 2), "GBps": gb(res["kernel_us"], alg_bytes),
+                         "pct_of_peak": round(gb(res["kernel_us"], alg_bytes) / 80, 2),
+                         "pct_of_load_pipeline": round(100 * res["load_pipeline_us"] / res["kernel_us"], 1)},
+        "n_gpus": 1, "steps": n_iter,
+    }), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -178,19 +261,25 @@ def main():
     torch.cuda.set_device(dev)
     if args.op == "kv_append":
         return bench_kv_append(args)
+    if args.op == "ceiling":
+        return bench_ceiling(args)
     t_gen = time.perf_counter()
     inp_cpu = wl.make_inputs(args.config)
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
     inp = inp_cpu.to(dev)
     pools = [(inp.k_cache, inp.v_cache)]
-    for r in range(1, max(1, args.rotate)):
+    pool_bytes = 2 * inp.k_cache.numel() * inp.k_cache.element_size()
+    rotate = max(1, args.rotate)
+    if args.rotate > 1:
+        rotate = max(rotate, min(16, -(-(1 << 30) // max(pool_bytes, 1))))       # small pools: more of them
+    for r in range(1, rotate):
         # further pools: same pages, different (seeded) contents - the access pattern is identical
         g = torch.Generator(device=dev).manual_seed(inp.cfg.seed + 100 * r)
         if inp.cfg.kv_dtype == "fp8_e4m3":
             mk = lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
                 torch.float8_e4m3fn)
         else:
-            mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=torch.bfloat16)
+            mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype)
         pools.append((mk(), mk()))
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
@@ -229,24 +318,71 @@ def main():
     gbps = alg_bytes / (wall_s / args.steps) / 1e9
 
     # ---- dominant kernel alone (split-KV), HIP events on the launch stream ------------------------------------
+    # A single-pass plan runs one kernel, the variant that writes (out, lse) itself: the events go around the call.
+    # A split plan runs the split kernel and the combine: the events go around the split launches only.
+    single_pass = plan.num_splits == 1
+    kernel_step = (lambda i: calls[i % len(calls)].run()) if single_pass else \
+        (lambda i: calls[i % len(calls)].run_splitkv())
     for i in range(min(args.warmup, 10)):
-        calls[i % len(calls)].run_splitkv()
+        kernel_step(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     e0.record()
     for i in range(args.steps):
-        calls[i % len(calls)].run_splitkv()
+        kernel_step(i)
     e1.record()
     torch.cuda.synchronize()
     split_us = e0.elapsed_time(e1) * 1e3 / args.steps
     split_gbps = alg_bytes / (split_us * 1e-6) / 1e9
 
+    # ---- the same calls replayed from one HIP graph (a serving engine replays its decode step from a graph):
+    # separates what the host-side launches cost from what the GPU needs
+    graph_us = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for c in calls:
+                c.run()                            # first use of the stream outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for c in calls:
+                c.run()
+        reps = max(1, args.steps // len(calls))
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_us = (time.perf_counter() - t0) * 1e6 / (reps * len(calls))
+
+    # ---- the un-prepared public entry point: flash_decode() validates, marshals and allocates (out, lse) per call
+    kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo,
+              max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+    n_entry = min(args.steps, 100)
+    for i in range(5):
+        tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens, inp.sm_scale, **kw)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(n_entry):
+        tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens, inp.sm_scale, **kw)
+    torch.cuda.synchronize()
+    entry_us = (time.perf_counter() - t0) * 1e6 / n_entry
+
     traffic = None
+    traffic_source = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
             traffic = json.load(f).get(args.config, {}).get("bytes_per_launch")
+        if traffic is not None:
+            traffic_source = "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run, not this one)"
 
+    qd = inp.cfg.q_dtype
     result = {
         "metric": "decode-attn achieved HBM GB/s (algorithmic bytes / time per call; µs/call alongside), "
                   "Llama-3-8B shape b=32" if args.config == "llama3_8b_b32" else f"decode-attn achieved HBM GB/s, {args.config}",
@@ -254,6 +390,8 @@ def main():
         "unit": "GB/s",
         "us_per_call": round(ms_per_step * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "graph_replay_us_per_call": None if graph_us is None else round(graph_us, 2),
+        "public_entry_us_per_call": round(entry_us, 2),
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
@@ -261,25 +399,29 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if inp.cfg.kv_dtype == "bf16" else "fp8_e4m3 KV / bf16 q, fp32 softmax",
-        "data": "synthetic (seeded N(0,1) bf16 q/K/V generated on the CPU, resident in HBM before timing)",
+        "dtype": qd if inp.cfg.kv_dtype != "fp8_e4m3" else f"fp8_e4m3 KV / {qd} q, fp32 softmax",
+        "data": f"synthetic, resident in HBM before timing: seeded N(0,1) {qd} q/K/V generated on the CPU" +
+                (f"; the timed calls cycle through {len(pools)} KV pools with the same block_table, pools 2.. filled on "
+                 "the GPU (seeded N(0,1), fp8: uniform codes 0..119)" if len(pools) > 1 else ""),
         "config": {
             "workload": f"{args.config}: {inp.cfg.description}",
             "algorithmic_bytes_per_call": alg_bytes,
             "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
-            "kv_pools_rotated": len(pools),
+            "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
             "host_length_hints": [min(inp.kv_lens_host), max(inp.kv_lens_host)],
         },
         "roofline": {
             "bound": "hbm",
             "kernel": f"splitkv_{plan.algo}_kernel",
+            "variant": "single pass: writes (out, lse) itself" if single_pass else "writes fp32 partials; the combine kernel follows",
             "achieved": round(split_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(split_gbps / HBM_PEAK_GBPS, 4),
             "us_per_launch": round(split_us, 2),
             "traffic": traffic,
+            "traffic_source": traffic_source,
         },
     }
     if not args.no_cpu_baseline:

@@ -637,6 +637,21 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
     # against the oracle's restatement of the reference merge
     want = cf.combine_ranks(outs.cpu(), lses.cpu(), shard_lens)
     torch.testing.assert_close(final2.double().cpu(), want, atol=4e-3, rtol=1e-2)
+    # the merged lse: the log-sum-exp of the ranks that hold tokens (sequence 2 has tokens on rank 3 only)
+    lse_out = torch.full((b, hq), float("nan"), dtype=torch.float32, device=cuda_device)
+    tda.inter_rank_combine(outs, gl, all_ranks_lse=lses, lse_out=lse_out)
+    torch.cuda.synchronize()
+    masked = torch.where((shard_lens > 0)[:, :, None].to(cuda_device), lses, torch.full_like(lses, float("-inf")))
+    torch.testing.assert_close(lse_out, torch.logsumexp(masked.double(), dim=0).float(), atol=1e-4, rtol=0)
+    # output tensors of the wrong dtype / shape / device are refused before anything is launched
+    for bad in (torch.empty(b, hq, dtype=torch.bfloat16, device=cuda_device),
+                torch.empty(b, hq - 1, dtype=torch.float32, device=cuda_device),
+                torch.empty(b, hq, dtype=torch.float32)):
+        with pytest.raises(ValueError):
+            tda.inter_rank_combine(outs, gl, all_ranks_lse=lses, lse_out=bad)
+    with pytest.raises(ValueError):
+        tda.inter_rank_combine(outs, gl, torch.empty(b, hq, d - 1, dtype=torch.bfloat16, device=cuda_device),
+                               all_ranks_lse=lses)
 
 
 # ---- large batches: single pass with blocks of 4 or 8 kv heads per (eight-wave) workgroup ------------------------------
@@ -1066,7 +1081,7 @@ def test_fp8_every_byte_value_dequantises_exactly(cuda_device, algo):
 _INPUT_CACHE = {}
 
 
-def _full_config(name, cuda_device, algo="auto"):
+def _full_config(name, cuda_device, algo="auto", **hints):
     if name not in _INPUT_CACHE:
         _INPUT_CACHE.clear()                         # one configuration resident at a time
         print(f"config {name}: generating", flush=True)
@@ -1074,9 +1089,9 @@ def _full_config(name, cuda_device, algo="auto"):
     inp = _INPUT_CACHE[name]
     print(f"config {name}: decode ({algo})", flush=True)
     out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
-                                k_scale=inp.k_scale, v_scale=inp.v_scale, algo=algo)
+                                k_scale=inp.k_scale, v_scale=inp.v_scale, algo=algo, **hints)
     torch.cuda.synchronize()
-    assert out.shape == inp.q.shape and out.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    assert out.shape == inp.q.shape and out.dtype == inp.q.dtype and lse.dtype == torch.float32
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
     return inp, out, lse
 
@@ -1128,3 +1143,28 @@ def test_config4_long_131k(cuda_device, algo):
 def test_config5_fp8_70b_b128(cuda_device, algo):
     inp, out, lse = _full_config("fp8_70b_b128", cuda_device, algo)
     _check_rows(inp, out, lse, range(0, 128, 9) if algo == "auto" else [5, 100], "cfg5")
+
+
+def test_config4_long_131k_with_the_length_hints_of_the_benchmark(cuda_device):
+    # bench.py passes the host-known length bounds: equal bounds select per-sequence chunks instead of balanced shares
+    cfg = wl.CONFIGS["long_131k"]
+    hints = dict(max_kv_len=cfg.kv_len, min_kv_len=cfg.kv_len)
+    inp, out, lse = _full_config("long_131k", cuda_device, **hints)
+    plan = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, **hints)
+    assert not plan.balanced and plan.num_splits > 1
+    _check_rows(inp, out, lse, range(4), "cfg4 hinted")
+
+
+# ---- the shape of the reference's published figure (README.md:200-202; test_sp_decode_attn.py:203-220):
+# batch 1, 96 q / 12 kv heads, fp16, page size 1, local KV 8K ... 128K, at full size ----------------------------
+@pytest.mark.parametrize("name", wl.REF_SHAPE_ORDER)
+def test_reference_published_shape(cuda_device, name):
+    inp, out, lse = _full_config(name, cuda_device)
+    assert out.dtype == torch.float16 and out.shape == (1, 96, 128)
+    _check_rows(inp, out, lse, [0], name)
+    # what the reference's layer passes: 32 forced splits, packed output (sp_flash_decode_layer.py:62,100-110)
+    packed = tda.gqa_fwd_batch_decode_intra_rank(inp.q, inp.k_cache, inp.v_cache, None, [1], inp.kv_lens,
+                                                 inp.block_table, inp.sm_scale, kv_split=32)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(packed[..., :128].float(), out.float(), atol=2e-3, rtol=1e-2)
+    torch.testing.assert_close(packed[..., 128].float(), lse, atol=2e-2, rtol=1e-2)      # lse rounded to fp16

@@ -20,13 +20,13 @@ FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK
 # fdk_algo
 FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
 # flags
-FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN = 1, 2
+FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_PROBE_LOADS = 1, 2, 4
 FDK_STATIC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (
     "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
     "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len", "fdk_kv_append",
-    "fdk_decode_static",
+    "fdk_decode_static", "fdk_probe_linear_read",
 )
 
 
@@ -133,6 +133,8 @@ def load() -> C.CDLL:
     lib.fdk_counters_len.argtypes = [C.POINTER(FdkDecodeArgs)]
     lib.fdk_combine_ranks.restype = C.c_int
     lib.fdk_combine_ranks.argtypes = [C.POINTER(FdkCombineRanksArgs), C.c_void_p]
+    lib.fdk_probe_linear_read.restype = C.c_int
+    lib.fdk_probe_linear_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
     lib.fdk_kv_append.restype = C.c_int
     lib.fdk_kv_append.argtypes = [C.POINTER(FdkKvAppendArgs), C.c_void_p]
     if lib.fdk_abi_version() != FDK_ABI_VERSION:

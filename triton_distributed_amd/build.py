@@ -22,7 +22,7 @@ OBJ_DIR = PKG_DIR / "build"
 SOURCES = [
     "fdk_api.hip", "fdk_combine.hip", "fdk_splitkv_valu.hip", "fdk_splitkv_mfma.hip",
     "fdk_splitkv_valu_bf16.hip", "fdk_splitkv_valu_bf16_fp8.hip", "fdk_splitkv_valu_fp16.hip",
-    "fdk_splitkv_valu_fp16_fp8.hip", "fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip", "fdk_kv_append.hip",
+    "fdk_splitkv_valu_fp16_fp8.hip", "fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip", "fdk_kv_append.hip", "fdk_probe.hip",
 ]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not to be generated for this target.

@@ -146,6 +146,12 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     // the kernels keep the byte offsets of a tile's 16 token rows relative to its first row in 32 bits
     if (a->k_stride_tok * kes * 16 >= ((int64_t)1 << 32) || a->v_stride_tok * kes * 16 >= ((int64_t)1 << 32))
         return fail(FDK_ESHAPE, "cache token stride too large: 16 rows must span less than 4 GiB");
+    // page number x page stride is a 32 x 32 -> 64 bit product in the kernels; token-in-page offsets are 32 bit
+    if (a->k_stride_page * kes >= ((int64_t)1 << 32) || a->v_stride_page * kes >= ((int64_t)1 << 32))
+        return fail(FDK_ESHAPE, "cache page stride too large: a page must span less than 4 GiB");
+    if ((int64_t)a->page_size * a->k_stride_tok * kes >= ((int64_t)1 << 32) ||
+        (int64_t)a->page_size * a->v_stride_tok * kes >= ((int64_t)1 << 32))
+        return fail(FDK_ESHAPE, "page_size x token stride must be less than 4 GiB");
     if (a->kv_dtype == FDK_FP8_E4M3 &&
         ((reinterpret_cast<uintptr_t>(a->k_scale) & 3u) || (reinterpret_cast<uintptr_t>(a->v_scale) & 3u)))
         return fail(FDK_EALIGN, "k_scale / v_scale must be 4-byte aligned");
@@ -328,6 +334,9 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
+    sp.probe = (a->flags & FDK_FLAG_PROBE_LOADS) ? 1 : 0;
+    if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128 || a->kv_dtype == FDK_FP8_E4M3))
+        return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path, head_dim 128, 16-bit cache");
     sp.scale_log2 = a->sm_scale * fdk::kLog2e;
     sp.soft_cap = a->soft_cap > 0.f ? a->soft_cap : 0.f;
     sp.sm_scale = a->sm_scale;
@@ -378,7 +387,7 @@ int decode_impl(const fdk_decode_args* args, void* hip_stream) {
     if (dry) return FDK_OK;
     rc = launch_split(args, r, stream);
     if (rc) return rc;
-    if (!r.sp.direct) {
+    if (!r.sp.direct && !r.sp.probe) {
         rc = fdk::launch_combine(r.cp, stream);
         if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
@@ -514,6 +523,17 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
     p.partial_dtype = a->partial_dtype; p.out_dtype = a->out_dtype; p.packed = packed ? 1 : 0;
     int rc = fdk::launch_combine_ranks(p, reinterpret_cast<hipStream_t>(hip_stream));
     if (rc) return fail(rc, "rank combine launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
+int fdk_probe_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, void* hip_stream) {
+    g_err[0] = 0;
+    if (!buf) return fail(FDK_ENULL, "buf is null");
+    if (!aligned16(buf)) return fail(FDK_EALIGN, "buf must be 16-byte aligned");
+    if (bytes < 65536) return fail(FDK_ESHAPE, "bytes %zu: at least 64 KB", bytes);
+    if (workgroups <= 0 || workgroups > (1 << 20)) return fail(FDK_ESHAPE, "workgroups %d outside [1, 2^20]", workgroups);
+    int rc = fdk::launch_linear_read(buf, bytes, nontemporal, workgroups, reinterpret_cast<hipStream_t>(hip_stream));
+    if (rc) return fail(rc, "linear read launch failed: %s", hipGetErrorString((hipError_t)rc));
     return FDK_OK;
 }
 

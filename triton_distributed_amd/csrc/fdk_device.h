@@ -45,6 +45,7 @@ struct SplitParams {
     int32_t persistent, total_items, num_cus;
     int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
+    int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     float scale_log2;               // sm_scale * log2(e)
     float soft_cap;                 // > 0: on (applied to natural-unit logits)
     float sm_scale;
@@ -107,6 +108,8 @@ struct KvAppendParams {
 int launch_kv_append(const KvAppendParams& p, int qkv_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
+int launch_splitkv_mfma_probe(const SplitParams& p, hipStream_t stream);      // head_dim 128, 16-bit cache
+int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream);
 int launch_combine(const CombineParams& p, hipStream_t stream);
 int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
 bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);

@@ -1,0 +1,64 @@
+// Measurement aids: what the memory system of this GPU delivers, with no arithmetic in the way.
+//   launch_splitkv_mfma_probe  the matrix-core split kernel reduced to its load pipeline (same pieces, same
+//                              addresses, same instructions in the same order) for head_dim 128 and a 16-bit cache
+//   launch_linear_read         a plain streaming read of a buffer, with or without the non-temporal hint
+// Neither produces results; bench.py --op ceiling times them next to the real kernels.
+#include "fdk_splitkv_mfma.h"
+
+namespace fdk {
+
+namespace {
+
+template <bool NT>
+__global__ __launch_bounds__(256) void linear_read_kernel(const u32x4_t* __restrict__ p, size_t n16, uint32_t* sink_out) {
+    // all workgroups sweep one moving window: 32 KB per workgroup and step, two steps in flight
+    constexpr int U = 8;
+    const size_t blk = 256 * U;
+    const size_t step = (size_t)gridDim.x * blk;
+    size_t i = (size_t)blockIdx.x * blk + threadIdx.x;
+    uint32_t acc = 0;
+    u32x4_t a[U], b[U];
+    auto ld = [&](const u32x4_t* q) { return NT ? __builtin_nontemporal_load(q) : *q; };
+    auto fits = [&](size_t at) { return at + 256 * (U - 1) < n16; };
+    if (fits(i)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) a[u] = ld(p + i + 256 * u);
+    }
+    for (; fits(i); i += 2 * step) {
+        const bool h1 = fits(i + step), h2 = fits(i + 2 * step);
+        if (h1) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) b[u] = ld(p + i + step + 256 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= a[u].x ^ a[u].y ^ a[u].z ^ a[u].w;
+        if (h2) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) a[u] = ld(p + i + 2 * step + 256 * u);
+        }
+        if (h1) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) acc ^= b[u].x ^ b[u].y ^ b[u].z ^ b[u].w;
+        }
+    }
+    if (acc == 0x9e3779b9u) *sink_out = acc;      // never true for real data; keeps the loads alive
+}
+
+}  // namespace
+
+int launch_splitkv_mfma_probe(const SplitParams& p, hipStream_t stream) {
+    if (p.head_dim != 128) return (int)hipErrorInvalidValue;
+    return launch_pm<FDK_BF16, false, 128, true>(p, stream);     // fp16 rows have the same bytes
+}
+
+int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream) {
+    const dim3 grid((unsigned)workgroups), block(256);
+    // the first 16 bytes of the buffer double as the (never written) checksum target
+    uint32_t* sink = reinterpret_cast<uint32_t*>(const_cast<void*>(buf));
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(buf);
+    if (nontemporal) hipLaunchKernelGGL(linear_read_kernel<true>, grid, block, 0, stream, p, bytes / 16, sink);
+    else hipLaunchKernelGGL(linear_read_kernel<false>, grid, block, 0, stream, p, bytes / 16, sink);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fdk

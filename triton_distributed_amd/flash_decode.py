@@ -242,7 +242,8 @@ class PreparedDecode:
 def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_cap=0.0, kv_split=-1,
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
-                   work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None) -> PreparedDecode:
+                   work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
+                   probe_loads=False) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -252,6 +253,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``work_queue=False`` launches one workgroup per item instead.
     ``stream_scratch``: a stream (handle); scratch that the call has to provide itself is then taken from a buffer
     kept per (device, stream) instead of a fresh allocation - only for calls that are issued on that stream at once.
+    ``probe_loads=True`` is a measurement aid: the call runs only the load pipeline of the split kernel (the same
+    pieces and addresses, no arithmetic, no combine) and leaves out / lse undefined.
     ``static_scratch=True`` binds no workspace and no counters: the call is then to be issued with
     ``run_static()``, which keeps the split partials in the library's own static scratch."""
     if not isinstance(kv_lens, torch.Tensor):
@@ -260,6 +263,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    k_scale, v_scale, algo, min_kv_len=min_kv_len)
     batch, q_heads, d = q.shape
     plan = _plan_of(a)
+    if probe_loads:
+        a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
         if tuple(packed_out.shape) != (batch, q_heads, d + 1) or packed_out.stride(-1) != 1:
             raise ValueError(f"packed output must be [B, Hq, D+1] = {(batch, q_heads, d + 1)}")
@@ -601,3 +606,12 @@ def qk_norm_rope_update_kvcache(qkv: torch.Tensor, key_cache: torch.Tensor, valu
     a.q_out_stride_b, a.q_out_stride_t, a.q_out_stride_h = q_norm_rope.stride(0), q_norm_rope.stride(1), q_norm_rope.stride(2)
     _lib.check(_LIB.fdk_kv_append(C.byref(a), _stream_handle(stream)))
     return q_norm_rope
+
+
+def probe_linear_read(buf: torch.Tensor, nontemporal: bool = True, workgroups: int = 512, stream=None) -> None:
+    """Measurement aid: stream ``buf`` (a contiguous GPU tensor) through ``workgroups`` workgroups once, with
+    16-byte loads that carry the non-temporal hint or not; nothing is written (``fdk_probe_linear_read``)."""
+    if not buf.is_cuda or not buf.is_contiguous():
+        raise ValueError("buf must be a contiguous GPU tensor")
+    _lib.check(_LIB.fdk_probe_linear_read(buf.data_ptr(), buf.numel() * buf.element_size(), int(bool(nontemporal)),
+                                          int(workgroups), _stream_handle(stream)))

@@ -28,7 +28,8 @@ class DecodeConfig:
     kv_len: Optional[int] = None         # uniform length, or
     kv_len_range: Optional[tuple] = None  # (lo, hi) inclusive, drawn per sequence
     q_scale: float = 1.0
-    kv_dtype: str = "bf16"               # "bf16" | "fp8_e4m3"
+    kv_dtype: str = "bf16"               # "bf16" | "fp16" | "fp8_e4m3"; a 16-bit cache has q's dtype
+    q_dtype: str = "bf16"                # "bf16" | "fp16"
     spare_pages: int = 64
     description: str = ""
 
@@ -46,6 +47,16 @@ CONFIGS: Dict[str, DecodeConfig] = {
                                  description="B128 64q/8kv D128 N8192 P16, e4m3 KV with per-kv-head scales"),
 }
 CONFIG_ORDER: List[str] = ["tiny", "llama3_8b_b32", "ragged_g8", "long_131k", "fp8_70b_b128"]
+
+# The shape behind the reference's only published figure for this path (README.md:200-202; perf loops of
+# test/nvidia/test_sp_decode_attn.py:203-220 and test_decode_attn.py:294-527): batch 1, 96 q / 12 kv heads,
+# head_dim 128, fp16, page size 1, local KV 8K ... 128K.
+REF_SHAPE_LENGTHS = {"8k": 8192, "16k": 16384, "32k": 32768, "64k": 65536, "128k": 131072}
+for _tag, _n in REF_SHAPE_LENGTHS.items():
+    CONFIGS[f"ref_b1_96q12kv_p1_{_tag}"] = DecodeConfig(
+        f"ref_b1_96q12kv_p1_{_tag}", 1100 + _n // 8192, 1, 96, 12, 128, 1, kv_len=_n, kv_dtype="fp16", q_dtype="fp16",
+        description=f"B1 96q/12kv D128 N{_n} P1 fp16 (the reference's published perf shape)")
+REF_SHAPE_ORDER: List[str] = [f"ref_b1_96q12kv_p1_{t}" for t in REF_SHAPE_LENGTHS]
 
 
 @dataclass
@@ -104,13 +115,13 @@ def quantize_kv_fp8(cache: torch.Tensor, chunk_pages: int = 4096):
     return out, scale
 
 
-def _randn_bf16(shape, gen: torch.Generator, chunk: int = 1 << 24) -> torch.Tensor:
-    """Seeded N(0,1) in bf16, drawn in fp32 pieces to bound peak memory."""
+def _randn_bf16(shape, gen: torch.Generator, chunk: int = 1 << 24, dtype=torch.bfloat16) -> torch.Tensor:
+    """Seeded N(0,1) in bf16 (or ``dtype``), drawn in fp32 pieces to bound peak memory."""
     n = math.prod(shape)
-    out = torch.empty(n, dtype=torch.bfloat16)
+    out = torch.empty(n, dtype=dtype)
     for lo in range(0, n, chunk):
         m = min(chunk, n - lo)
-        out[lo:lo + m] = torch.randn(m, generator=gen, dtype=torch.float32).to(torch.bfloat16)
+        out[lo:lo + m] = torch.randn(m, generator=gen, dtype=torch.float32).to(dtype)
     return out.view(shape)
 
 
@@ -139,12 +150,13 @@ def make_inputs(name_or_cfg, device="cpu", poison_tail: bool = False) -> DecodeI
     for b, n_pg in enumerate(pages_per_seq):
         table[b, :n_pg] = perm[pos:pos + n_pg]
         pos += n_pg
-    q = _randn_bf16((cfg.batch, cfg.q_heads, cfg.head_dim), gen)
+    dt = torch.float16 if cfg.q_dtype == "fp16" else torch.bfloat16
+    q = _randn_bf16((cfg.batch, cfg.q_heads, cfg.head_dim), gen, dtype=dt)
     if cfg.q_scale != 1.0:
-        q = (q.float() * cfg.q_scale).to(torch.bfloat16)
+        q = (q.float() * cfg.q_scale).to(dt)
     cache_shape = (pool, cfg.page_size, cfg.kv_heads, cfg.head_dim)
-    k_cache = _randn_bf16(cache_shape, gen)
-    v_cache = _randn_bf16(cache_shape, gen)
+    k_cache = _randn_bf16(cache_shape, gen, dtype=dt)
+    v_cache = _randn_bf16(cache_shape, gen, dtype=dt)
     k_scale = v_scale = None
     if cfg.kv_dtype == "fp8_e4m3":
         k_cache, k_scale = quantize_kv_fp8(k_cache)
@@ -159,5 +171,5 @@ def scaled_down(cfg: DecodeConfig, batch: Optional[int] = None, kv_len: Optional
     """Same layout, smaller extent (for CPU-sized checks)."""
     return DecodeConfig(cfg.name + "_small", cfg.seed, batch or cfg.batch, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
                         cfg.page_size, kv_len if cfg.kv_len is not None else None,
-                        kv_len_range if cfg.kv_len is None else None, cfg.q_scale, cfg.kv_dtype,
+                        kv_len_range if cfg.kv_len is None else None, cfg.q_scale, cfg.kv_dtype, cfg.q_dtype,
                         min(cfg.spare_pages, 8), cfg.description)
