@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
+    ap.add_argument("--single-launch", action="store_true",
+                    help="split plans: let the last workgroup of a (sequence, head block) merge the partials instead "
+                         "of launching the combine kernel (FDK_FLAG_SINGLE_LAUNCH; slower on MI355X, for comparison)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
@@ -283,7 +286,8 @@ def main():
         pools.append((mk(), mk()))
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
-                                max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+                                max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host),
+                                single_launch=args.single_launch)
              for k, v in pools]
     plan = calls[0].plan
     alg_bytes = inp.algorithmic_bytes()
@@ -408,6 +412,7 @@ def main():
             "algorithmic_bytes_per_call": alg_bytes,
             "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
+            "single_launch": bool(args.single_launch and plan.num_splits > 1),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
             "host_length_hints": [min(inp.kv_lens_host), max(inp.kv_lens_host)],
         },

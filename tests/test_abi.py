@@ -181,7 +181,7 @@ def test_counters_of_the_work_queue_form():
     lib = _lib.load()
     a = _args(batch=4)
     n = lib.fdk_counters_len(C.byref(a))
-    assert n == 2
+    assert n == 2 + 4 * 8          # queue head, finished workgroups, a ticket per (sequence, kv head, head tile)
     assert lib.fdk_counters_len(None) == 0
     a.counters, a.counters_len = 0x90000, n
     assert _decode_rc(a) == 0

@@ -466,22 +466,30 @@ def test_split_then_combine_entry_points_equal_the_fused_call(cuda_device):
 
 @pytest.mark.parametrize("config,kw", [("ragged_g8", dict(batch=40, kv_len_range=(1, 6000))),
                                        ("llama3_8b_b32", dict(batch=3, kv_len=3000))])
-def test_work_queue_form_equals_one_workgroup_per_item_and_restores_its_counters(cuda_device, config, kw):
-    # a fixed set of workgroups pulling items from a queue against one workgroup per item
+def test_single_launch_form_equals_split_then_combine_and_restores_its_counters(cuda_device, config, kw):
+    # with counters: one launch (the last workgroup of a unit merges; many pieces are pulled from a queue) against
+    # one workgroup per piece followed by the combine kernel
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS[config], **kw), cuda_device, poison_tail=True)
     for kv_split in (-1, 7, 64):
         two = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
                                  kv_split=kv_split, work_queue=False)
-        ctr = torch.zeros(8, dtype=torch.int32, device=cuda_device)
+        ctr = torch.zeros(4096, dtype=torch.int32, device=cuda_device)
         one = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
-                                 kv_split=kv_split, counters=ctr)
-        assert one.plan.num_splits == two.plan.num_splits
+                                 kv_split=kv_split, counters=ctr, single_launch=True)
+        assert one.plan.num_splits == two.plan.num_splits and one.args.counters and not two.args.counters
         o2, l2 = two.run()
+        firsts = None
         for _ in range(3):                               # repeated calls reuse the same counters
-            one.out.zero_()
+            one.out.fill_(float("nan"))
+            one.lse.fill_(float("nan"))
             o1, l1 = one.run()
-        torch.cuda.synchronize()
-        assert torch.equal(o1, o2) and torch.equal(l1, l2)     # same items, same arithmetic, same merge
+            torch.cuda.synchronize()
+            if firsts is None:
+                firsts = (o1.clone(), l1.clone())
+            assert torch.equal(o1, firsts[0]) and torch.equal(l1, firsts[1])      # whoever merges: same arithmetic
+        # same pieces; the two merges differ in rounding only (at most one step of the 16-bit output)
+        torch.testing.assert_close(o1.float(), o2.float(), atol=2e-3, rtol=2 ** -7)
+        torch.testing.assert_close(l1, l2, atol=2e-6, rtol=1e-6)
         assert int(ctr.abs().sum()) == 0
         _check(o1, l1, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
                tag=f"work queue S={kv_split}")
@@ -1168,3 +1176,74 @@ def test_reference_published_shape(cuda_device, name):
     torch.cuda.synchronize()
     torch.testing.assert_close(packed[..., :128].float(), out.float(), atol=2e-3, rtol=1e-2)
     torch.testing.assert_close(packed[..., 128].float(), lse, atol=2e-2, rtol=1e-2)      # lse rounded to fp16
+
+
+# ---- single launch: the last workgroup of a (sequence, head block, head tile) merges its pieces ----------------------
+# (the reference's persistent kernel merges after a grid barrier, flash_decode.py:719-760)
+FUSED_CASES = {
+    # name: (batch, hq, hkv, head_dim, page, kv_lens or (lo, hi), kv dtype, kv_split)
+    "chunks_short": (3, 32, 8, 128, 16, [700, 64, 1], torch.bfloat16, -1),
+    "chunks_forced_32": (5, 32, 8, 128, 16, [4000, 1, 17, 2049, 333], torch.bfloat16, 32),
+    "chunks_more_splits_than_tokens": (2, 8, 2, 128, 1, [5, 70], torch.float16, 64),
+    "queue_many_items": (12, 32, 8, 128, 16, (1, 3000), torch.bfloat16, 24),
+    "balanced_ragged": (9, 8, 1, 128, 16, [30000, 1, 0, 777, 12000, 64, 65, 0, 5000], torch.bfloat16, -1),
+    "balanced_all_but_one_empty": (4, 16, 2, 128, 16, [0, 0, 70000, 0], torch.bfloat16, -1),
+    "balanced_two_tiles_d64": (3, 48, 2, 64, 16, [40000, 60000, 40], torch.float16, -1),
+    "balanced_fp8_d256": (2, 16, 4, 256, 16, [60000, 30000], "fp8", -1),
+    "ref_shape_p1": (1, 96, 12, 128, 1, [6000], torch.float16, -1),
+}
+
+
+@pytest.mark.parametrize("name", list(FUSED_CASES))
+def test_single_launch_decode_against_the_oracle_and_the_two_launch_form(cuda_device, name):
+    batch, hq, hkv, d, page, lens, dt, kv_split = FUSED_CASES[name]
+    g = torch.Generator().manual_seed(sum(map(ord, name)))
+    if isinstance(lens, tuple):
+        lens = torch.randint(lens[0], lens[1] + 1, (batch,), generator=g).tolist()
+    fp8 = dt == "fp8"
+    qdt = torch.bfloat16 if fp8 else dt
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 4
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, max(max(pages), 1)), -1, dtype=torch.int32)        # poison: never used as a page
+    pos = 0
+    for b, n_pg in enumerate(pages):
+        table[b, :n_pg] = perm[pos:pos + n_pg]
+        pos += n_pg
+    q = torch.randn(batch, hq, d, generator=g).to(qdt).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(qdt)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(qdt)
+    ks = vs = None
+    ref_kv = None
+    if fp8:
+        k8, ks = wl.quantize_kv_fp8(k)
+        v8, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k8, ks).to(cuda_device), ofp8.dequant_per_head(v8, vs).to(cuda_device))
+        k, v, ks, vs = k8, v8, ks.to(cuda_device), vs.to(cuda_device)
+    k, v, table = k.to(cuda_device), v.to(cuda_device), table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    scale = d ** -0.5
+    kw = dict(kv_split=kv_split, k_scale=ks, v_scale=vs, max_kv_len=max(max(lens), 1))
+    two = tda.prepare_decode(q, k, v, table, lens_t, scale, work_queue=False, **kw)
+    one = tda.prepare_decode(q, k, v, table, lens_t, scale, single_launch=True, **kw)
+    assert one.plan.num_splits > 1 and one.args.counters and not two.args.counters, one.plan
+    if name.startswith("balanced"):
+        assert one.plan.balanced
+    o2, l2 = [t.clone() for t in two.run()]
+    first = None
+    for it in range(25):                  # the merging workgroup changes from run to run; the result must not
+        one.out.fill_(float("nan"))
+        one.lse.fill_(float("nan"))
+        o1, l1 = one.run()
+        torch.cuda.synchronize()
+        if first is None:
+            first = (o1.clone(), l1.clone())
+        assert torch.equal(o1, first[0]) and torch.equal(l1, first[1]), f"{name}: run {it} differs from run 0"
+    live = [b for b in range(batch) if lens[b] > 0]
+    dead = [b for b in range(batch) if lens[b] == 0]
+    torch.testing.assert_close(o1[live].float(), o2[live].float(), atol=2e-3, rtol=2 ** -7)
+    torch.testing.assert_close(l1[live], l2[live], atol=2e-6, rtol=1e-6)
+    if dead:
+        assert torch.all(o1[dead] == 0) and torch.all(l1[dead] == float("-inf"))
+    _check(o1[live], l1[live], q[live], k, v, table[live], [lens[b] for b in live], scale, ref_kv=ref_kv, tag=name)
+    assert int(one._keep[-1].abs().sum()) == 0                  # the counters are back at zero

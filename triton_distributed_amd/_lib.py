@@ -20,7 +20,7 @@ FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK
 # fdk_algo
 FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
 # flags
-FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_PROBE_LOADS = 1, 2, 4
+FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_PROBE_LOADS, FDK_FLAG_SINGLE_LAUNCH = 1, 2, 4, 8
 FDK_STATIC_SCRATCH_BYTES = 32 << 20
 
 EXPORTS = (

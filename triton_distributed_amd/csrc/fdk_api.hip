@@ -375,19 +375,27 @@ int decode_impl(const fdk_decode_args* args, void* hip_stream) {
     rc = resolve(args, true, dry ? kDryRunCus : 0, &r);
     if (rc) return rc;
     hipStream_t stream = reinterpret_cast<hipStream_t>(hip_stream);
-    // work-queue form of the split kernel (matrix-core path only)
-    const bool queued = !r.sp.direct && !r.sp.balanced && args->counters != nullptr && r.plan.algo == FDK_ALGO_MFMA;
-    if (queued) {
+    // With counters (matrix-core path only): a forced split count with more items than are resident at once runs
+    // as a work queue; and with FDK_FLAG_SINGLE_LAUNCH the workgroup that finishes a (sequence, head block,
+    // head tile) last merges its pieces, so no combine launch follows.
+    const bool with_counters = !r.sp.direct && !r.sp.probe && args->counters != nullptr && r.plan.algo == FDK_ALGO_MFMA;
+    if (with_counters) {
         if (reinterpret_cast<uintptr_t>(args->counters) & 3u) return fail(FDK_EALIGN, "counters not 4-byte aligned");
         if (args->counters_len < fdk_counters_len(args))
             return fail(FDK_EWORKSPACE, "counters_len %lld < %lld", (long long)args->counters_len,
                         (long long)fdk_counters_len(args));
         r.sp.counters = args->counters;
+        // the merging workgroup addresses the partials with 32-bit offsets
+        const size_t ws_need = fdk_workspace_bytes(args->batch, args->num_q_heads, args->head_dim, r.plan.num_splits);
+        if ((args->flags & FDK_FLAG_SINGLE_LAUNCH) && ws_need < ((size_t)1 << 32)) {
+            r.sp.fused = 1;
+            r.sp.ws_bytes = (uint32_t)ws_need;
+        }
     }
     if (dry) return FDK_OK;
     rc = launch_split(args, r, stream);
     if (rc) return rc;
-    if (!r.sp.direct && !r.sp.probe) {
+    if (!r.sp.direct && !r.sp.probe && !r.sp.fused) {
         rc = fdk::launch_combine(r.cp, stream);
         if (rc) return fail(rc, "combine kernel launch failed: %s", hipGetErrorString((hipError_t)rc));
     }
@@ -405,8 +413,11 @@ const char* fdk_last_error(void) { return g_err; }
 int fdk_device_cus(void) { return query_cus(); }
 
 int64_t fdk_counters_len(const fdk_decode_args* a) {
-    if (!a || a->batch <= 0 || a->num_q_heads <= 0) return 0;
-    return 2;      // queue head, finished-workgroup count
+    if (!a || a->batch <= 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads) return 0;
+    // queue head, finished-workgroup count, then one ticket per (sequence, kv head, tile of 16 q heads): an upper
+    // bound of the (sequence, head block, head tile) units of any plan
+    const int64_t group = a->num_q_heads / a->num_kv_heads;
+    return 2 + (int64_t)a->batch * a->num_kv_heads * ((group + 15) / 16);
 }
 
 size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim, int32_t num_splits) {

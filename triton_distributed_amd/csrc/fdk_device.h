@@ -46,6 +46,9 @@ struct SplitParams {
     int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
+    uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
+    int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its
+                                    // pieces into (out, lse); tickets at counters[2 + ...], no combine launch
     float scale_log2;               // sm_scale * log2(e)
     float soft_cap;                 // > 0: on (applied to natural-unit logits)
     float sm_scale;

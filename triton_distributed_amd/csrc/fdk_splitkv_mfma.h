@@ -90,6 +90,126 @@ __device__ __forceinline__ void put(uint32_t (&dst)[4], const uint4 x) {
 }
 __device__ __forceinline__ uint4 get(const uint32_t (&src)[4]) { return make_uint4(src[0], src[1], src[2], src[3]); }
 
+// ---- partial rows that another workgroup of the same launch merges (fused combine) ----------------------------
+// The L2 caches of the eight XCDs are not coherent with each other.  Rows that cross workgroups are therefore
+// written and read with relaxed atomic accesses of agent scope (write-through stores, loads that do not hit
+// stale lines), which need no cache write-back or invalidation; the order "rows, then ticket" is enforced by
+// waiting for the stores before the ticket is drawn (ticket_arrive).
+__device__ __forceinline__ void st_agent2(float* p, float a, float b) {
+    const uint64_t v = (uint64_t)__builtin_bit_cast(uint32_t, a) | ((uint64_t)__builtin_bit_cast(uint32_t, b) << 32);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_agent1(float* p, float a) {
+    __hip_atomic_store(p, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Where the pieces of an output row are: piece s of (kv head hl of the block, head g of the tile) is partial row
+// base + s * piece_step + hl * hl_step + g * g_step; `live` pieces exist (each holds at least one token).
+struct MergeRows {
+    int64_t base, piece_step, hl_step, g_step;
+    int live;
+};
+
+// Log-sum-exp merge of the live pieces of up to NR output rows by one wavefront.  The rows go together so that
+// their loads are under way at the same time: a lane per piece loads the lse values, D / 4 lanes load a piece's row
+// 16 bytes each (64 / (D / 4) pieces per instruction), and the first batch of rows is requested before the
+// weights are known.  The loads bypass this XCD's L2 (sc1): the rows were written by workgroups on any XCD.
+template <int D, int NR>
+__device__ __forceinline__ void merge_rows(const SplitParams& p, const int64_t (&row0)[NR], const int (&hq)[NR], const int nrows,
+                                           const int64_t piece_step, const int live, const int b, const int lane) {
+    constexpr int LPR = D / 4;              // lanes per partial row
+    constexpr int PPI = 64 / LPR;           // pieces per load instruction
+    constexpr int NB = 8;                   // load instructions per row and batch
+    constexpr int kSc1 = 16;                // cache policy of the buffer loads: agent scope
+    const int sub = lane / LPR, col = lane % LPR;
+    const __amdgpu_buffer_rsrc_t ws = __builtin_amdgcn_make_buffer_rsrc(p.part_o, 0, (int)p.ws_bytes, 0x00020000);
+    const uint32_t lse_base = (uint32_t)((p.part_lse - p.part_o) * 4);
+    const uint32_t o_step = (uint32_t)(piece_step * D * 4), l_step = (uint32_t)(piece_step * 4);
+    f32x4_t acc[NR];
+    float m_run[NR], l_run[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        acc[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        m_run[r] = -INFINITY;
+        l_run[r] = 0.f;
+    }
+    for (int s0 = 0; s0 < live; s0 += 64) {             // blocks of 64 pieces: a lane per piece for the weights
+        const int n = min(64, live - s0);
+        float my[NR];
+        f32x4_t o[NR][NB];
+        auto request = [&](int t0) {                     // rows of pieces s0 + t0 + j * PPI + sub, j < NB
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                if (r < nrows) {
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) {
+                        const int t = t0 + j * PPI + sub;
+                        o[r][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                        if (t < n)
+                            o[r][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                ws, (uint32_t)(s0 + t) * o_step + col * 16, (uint32_t)(row0[r] * D * 4), kSc1));
+                    }
+                }
+            }
+        };
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            my[r] = -INFINITY;
+            if (r < nrows && lane < n)
+                my[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                            ws, (uint32_t)(s0 + lane) * l_step, lse_base + (uint32_t)(row0[r] * 4), kSc1)) * kLog2e;
+        }
+        request(0);
+        float w[NR];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            w[r] = 0.f;
+            if (r < nrows) {
+                const float m_new = fmaxf(m_run[r], wave_max(my[r]));      // finite: a live piece holds a token
+                w[r] = fast_exp2(my[r] - m_new);                           // 0 for idle lanes
+                const float alpha = fast_exp2(m_run[r] - m_new);
+                l_run[r] = l_run[r] * alpha + wave_sum(w[r]);
+                acc[r] *= alpha;
+                m_run[r] = m_new;
+            }
+        }
+        for (int t0 = 0; t0 < n; t0 += NB * PPI) {
+            if (t0 > 0) request(t0);
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                if (r < nrows) {
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) {
+                        const int t = min(t0 + j * PPI + sub, 63);
+                        acc[r] += __shfl(w[r], t, 64) * o[r][j];           // rows past the end were set to zero
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        if (r < nrows) {
+            f32x4_t a = acc[r];
+            if (PPI >= 2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[i] += __shfl_xor(a[i], 32, 64);
+            }
+            if (PPI >= 4) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[i] += __shfl_xor(a[i], 16, 64);
+            }
+            const float inv = fast_rcp(l_run[r]);
+            const float lse = (m_run[r] + fast_log2(l_run[r])) * kLn2;
+            const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq[r] * p.out_sh;
+            if (sub == 0) store_out4(p.out, ob + 4 * col, make_float4(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv), p.out_dtype);
+            if (lane == 0) {
+                if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq[r]] = lse;
+                if (p.pack_lse) store_out(p.out, ob + D, lse, p.out_dtype);
+            }
+        }
+    }
+}
+
 // PROBE: the load pipeline alone - the same pieces, addresses and load instructions in the same order, but what
 // arrives is only folded into a checksum: how fast the memory system serves this call's access pattern.
 template <int QDT, bool FP8, int PM, int NBUF, int D, bool PROBE = false>
@@ -127,8 +247,23 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     // ---- one piece of work: tokens [c_start, min(c_limit, kv_len)) of sequence b for kv-head block hgb and q-head
     // tile ht.  Partial results of head g of the tile go to row prow0 + g * prow_step of the workspace.
+    // out = 0, lse = -inf for the q heads [head0, head0 + heads_here) of an empty sequence; one wavefront
+    auto write_empty_rows = [&](const int b, const int head0, const int heads_here) {
+        for (int idx = lane; idx < heads_here * D; idx += 64) {
+            const int g = idx / D, d = idx % D;
+            const int64_t ob = (int64_t)b * p.out_sb + (int64_t)(head0 + g) * p.out_sh;
+            store_out(p.out, ob + d, 0.f, p.out_dtype);
+            if (d == 0) {
+                if (p.lse) p.lse[(int64_t)b * p.lse_sb + head0 + g] = -INFINITY;
+                if (p.pack_lse) store_out(p.out, ob + D, -INFINITY, p.out_dtype);
+            }
+        }
+    };
+
+    // With p.fused the workgroup that completes a (sequence, head block, head tile) - the last of its mr.live pieces
+    // to draw a ticket - merges the pieces into the final rows; no combine launch follows.
     auto run_piece = [&](const int b, const int hgb, const int ht, const int c_start, const int c_limit,
-                         const int64_t prow0, const int prow_step) {
+                         const int64_t prow0, const int prow_step, MergeRows mr) {
     const int kvh = hgb * nh + hl;
     const int head0 = kvh * p.group + ht * 16;
     const int heads_here = min(16, p.group - ht * 16);
@@ -150,20 +285,12 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     if (PM == PM_TILE) first_pg = tbl[min(c_start + tix * kTile, p.max_tokens - 1) >> p.page_shift];
     const int kv_len = min(p.kv_lens[b], p.max_tokens);
     if (c_start >= kv_len) {
-        if (p.direct && tix == 0) {   // kv_len == 0 with a single split: defined result, no combine follows
-            for (int idx = lane; idx < heads_here * D; idx += 64) {
-                const int g = idx / D, d = idx % D;
-                const int64_t ob = (int64_t)b * p.out_sb + (int64_t)(head0 + g) * p.out_sh;
-                store_out(p.out, ob + d, 0.f, p.out_dtype);
-                if (d == 0) {
-                    if (p.lse) p.lse[(int64_t)b * p.lse_sb + head0 + g] = -INFINITY;
-                    if (p.pack_lse) store_out(p.out, ob + D, -INFINITY, p.out_dtype);
-                }
-            }
-        }
+        // kv_len == 0: a defined result where no combine follows (the first piece writes it)
+        if ((p.direct || (p.fused && c_start == 0)) && tix == 0) write_empty_rows(b, head0, heads_here);
         return;
     }
     const int c_end = min(c_limit, kv_len);
+    if (!p.balanced) mr.live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);     // chunks that hold tokens
 
     float kscale = 1.f, vscale = 1.f;
     if (FP8) {
@@ -473,16 +600,50 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                 const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0;
                 store_out4(p.out, ob, o, p.out_dtype);
             } else {
-                const int64_t row = prow0 + (int64_t)c * prow_step;
-                *reinterpret_cast<float4*>(p.part_o + row * D + d0) = o;
+                float* dst = p.part_o + (prow0 + (int64_t)c * prow_step) * D + d0;
+                if (p.fused) {
+                    st_agent2(dst, o.x, o.y);
+                    st_agent2(dst + 2, o.z, o.w);
+                } else {
+                    *reinterpret_cast<float4*>(dst) = o;
+                }
             }
         }
         if (tix == 0 && a == 0) {
             if (p.direct) {
                 if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
                 if (p.pack_lse) store_out(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + D, lse_nat, p.out_dtype);
+            } else if (p.fused) {
+                st_agent1(p.part_lse + prow0 + (int64_t)c * prow_step, lse_nat);
             } else {
                 p.part_lse[prow0 + (int64_t)c * prow_step] = lse_nat;
+            }
+        }
+    }
+    if (p.fused && !p.direct) {
+        // rows first, then the ticket: every wave waits until its stores are done, the barrier collects the
+        // waves, one thread draws.  The last piece of the unit to arrive finds live - 1 and merges.
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        int* ticket = p.counters + 2 + (b * p.hg_blocks + hgb) * p.head_tiles + ht;
+        if (threadIdx.x == 0)
+            s_next[1] = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_next[1] == mr.live - 1) {
+            if (threadIdx.x == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            constexpr int NR = 2;                                     // rows a wavefront merges together
+            const int n_rows = nh * heads_here;
+            for (int r0 = wave * NR; r0 < n_rows; r0 += nw * NR) {
+                int64_t row0[NR];
+                int hq_of[NR];
+#pragma unroll
+                for (int i = 0; i < NR; ++i) {
+                    const int r = min(r0 + i, n_rows - 1);
+                    const int rh = r / heads_here, g = r % heads_here;
+                    row0[i] = mr.base + rh * mr.hl_step + g * mr.g_step;
+                    hq_of[i] = (hgb * nh + rh) * p.group + ht * 16 + g;
+                }
+                merge_rows<D, NR>(p, row0, hq_of, min(NR, n_rows - r0), mr.piece_step, mr.live, b, lane);
             }
         }
     }
@@ -513,8 +674,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         const int split = wg % p.num_splits;
         const int pb = wg / p.num_splits;
         // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
+        const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
         run_piece(pb, hgb, ht, split * p.chunk, split == p.num_splits - 1 ? p.max_tokens : split * p.chunk + p.chunk,
-                  ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split, p.num_splits);
+                  unit_row0 + (int64_t)hl * p.group * p.num_splits + split, p.num_splits,
+                  MergeRows{unit_row0, 1, (int64_t)p.group * p.num_splits, p.num_splits, 0});
         return;
     }
     const int units = p.hg_blocks * p.head_tiles;
@@ -523,14 +686,29 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     int x = 0, hi = 0;                            // balanced mode: next granule, end of this workgroup's share
     int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
     const int wc = blockIdx.x / units, bu = blockIdx.x % units;
+    int share_q = 1, share_r = 0;                 // balanced mode: granules per share, shares with one more
     if (p.balanced) {
         const int g_first = lane < p.batch ? granules_of(lane) : 0;          // sequences 0..63
         const int incl_first = wave_scan_i32(g_first);
         int total = __builtin_amdgcn_readlane(incl_first, 63);
         for (int b0 = 64; b0 < p.batch; b0 += 64) total += wave_sum_i32(b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
         const int shares = min((int)(gridDim.x / units), total);
+        if (p.fused && wc == 0 && tix == 0) {
+            // no piece, hence no merge, ever touches a sequence without tokens: the first share writes those rows
+            for (int b0 = 0; b0 < p.batch; b0 += 64) {
+                const int g = b0 == 0 ? g_first : (b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
+                uint64_t empty = __builtin_amdgcn_ballot_w64(b0 + lane < p.batch && g == 0);
+                for (; empty; empty &= empty - 1) {
+                    const int ht_e = bu % p.head_tiles;
+                    write_empty_rows(b0 + __builtin_ctzll(empty), ((bu / p.head_tiles) * nh + hl) * p.group + ht_e * 16,
+                                     min(16, p.group - ht_e * 16));
+                }
+            }
+        }
         if (wc >= shares) return;                                            // also total == 0
         const int q = total / shares, r = total % shares;
+        share_q = q;
+        share_r = r;
         x = wc * q + min(wc, r);
         hi = x + q + (wc < r ? 1 : 0);
         for (int b0 = 0, run = 0; b0 < p.batch; b0 += 64) {
@@ -554,6 +732,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         int pb, hgb, ht, c_start, c_limit, prow_step;
         int64_t prow0;
         int piece_end = 0;
+        MergeRows mr;
         if (p.balanced) {
             piece_end = min(before + gb, hi);
             pb = b;
@@ -564,6 +743,18 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             const int64_t slot = (int64_t)(wc + b) * units + bu;
             prow0 = slot * p.rows_per_slot + hl * p.heads_per_tile;
             prow_step = 1;
+            // the shares that hold granules [before, before + gb) of this sequence (the first share_r shares
+            // have share_q + 1 granules)
+            auto share_of = [&](int g) {
+                const int big = share_r * (share_q + 1);
+                return g < big ? g / (share_q + 1) : share_r + (g - big) / share_q;
+            };
+            const int wc_first = share_of(before);
+            mr.live = share_of(before + gb - 1) - wc_first + 1;
+            mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
+            mr.piece_step = (int64_t)units * p.rows_per_slot;
+            mr.hl_step = p.heads_per_tile;
+            mr.g_step = 1;
         } else {
             int wg = item;
             ht = wg % p.head_tiles;
@@ -576,6 +767,11 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + p.chunk;
             prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
             prow_step = p.num_splits;
+            mr.live = 0;                                              // from kv_len, inside run_piece
+            mr.base = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
+            mr.piece_step = 1;
+            mr.hl_step = (int64_t)p.group * p.num_splits;
+            mr.g_step = p.num_splits;
         }
         // everything that describes the piece is wave-uniform: keep it in scalar registers
         pb = __builtin_amdgcn_readfirstlane(pb);
@@ -586,7 +782,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         prow_step = __builtin_amdgcn_readfirstlane(prow_step);
         prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(prow0 >> 32)) << 32) |
                 (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)prow0);
-        run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step);
+        run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step, mr);
         if (p.balanced) {
             x = piece_end;
             if (x >= hi) return;

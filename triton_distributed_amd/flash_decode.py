@@ -170,7 +170,7 @@ def _capturing() -> bool:
     return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
 
 
-def _stream_counters(device: torch.device, stream, n: int = 64) -> Optional[torch.Tensor]:
+def _stream_counters(device: torch.device, stream, n: int) -> Optional[torch.Tensor]:
     """Zeroed int32 counters shared by the eager calls issued on one stream (they run in order, and every call
     leaves the counters zero), so the convenience entry points need no fill launch per call.  A call made while
     its stream is capturing a HIP graph gets counters of its own instead (None here: ``prepare_decode`` then
@@ -180,7 +180,7 @@ def _stream_counters(device: torch.device, stream, n: int = 64) -> Optional[torc
     key = (device.index, _stream_handle(stream))
     t = _COUNTER_CACHE.get(key)
     if t is None or t.numel() < n:
-        t = torch.zeros(n, dtype=torch.int32, device=device)
+        t = torch.zeros(max(n, 1024), dtype=torch.int32, device=device)
         _COUNTER_CACHE[key] = t
     return t
 
@@ -243,14 +243,19 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
-                   probe_loads=False) -> PreparedDecode:
+                   probe_loads=False, single_launch=False) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
     dtype) in ``[..., D]`` - the reference's ``output_combine`` layout - instead of ``out``.
-    ``counters``: zeroed int32 tensor for the work-queue form of a split decode (a fixed set of workgroups pulls
-    the work items, which keeps ragged batches balanced); by default the call owns a private one.
-    ``work_queue=False`` launches one workgroup per item instead.
+    ``counters``: zeroed int32 tensor (``fdk_counters_len`` elements) for the work-queue form of a split decode (a
+    forced split count with more pieces than fit the GPU at once: a fixed set of workgroups pulls the pieces, which
+    keeps ragged batches balanced) and for ``single_launch``; by default the call owns a private one (or, with
+    ``stream_scratch``, shares the stream's).  Every call leaves the counters zero.
+    ``work_queue=False`` launches one workgroup per piece instead.
+    ``single_launch=True``: no combine kernel - the workgroup that finishes a (sequence, head block) last merges the
+    partials (the reference's persistent kernel does this after a grid barrier, flash_decode.py:719-760).  Slower
+    than the two launches on MI355X, whose XCDs do not share an L2: measured, kept for comparison.
     ``stream_scratch``: a stream (handle); scratch that the call has to provide itself is then taken from a buffer
     kept per (device, stream) instead of a fresh allocation - only for calls that are issued on that stream at once.
     ``probe_loads=True`` is a measurement aid: the call runs only the load pipeline of the split kernel (the same
@@ -302,8 +307,12 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         a.workspace = workspace.data_ptr()
         a.workspace_bytes = workspace.numel() * workspace.element_size()
-    if plan.num_splits > 1 and plan.algo == "mfma" and work_queue and not plan.balanced:
+    if single_launch:
+        a.flags |= _lib.FDK_FLAG_SINGLE_LAUNCH
+    if plan.num_splits > 1 and plan.algo == "mfma" and ((work_queue and not plan.balanced) or single_launch):
         n_ctr = int(_LIB.fdk_counters_len(C.byref(a)))
+        if counters is None and stream_scratch is not None:
+            counters = _stream_counters(q.device, stream_scratch, n_ctr)         # None while capturing a graph
         if counters is None:
             counters = torch.zeros(n_ctr, dtype=torch.int32, device=q.device)
         elif counters.dtype != torch.int32 or counters.numel() < n_ctr or not counters.is_cuda or \
@@ -347,7 +356,6 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
                           out=out, lse=lse, workspace=workspace, algo=algo, min_kv_len=min_kv_len,
                           stream_scratch=stream if q.is_cuda else None,
-                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)
 
@@ -366,9 +374,7 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
-                          want_lse=False, stream_scratch=stream if q.is_cuda else None,
-                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
-                          work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
     call.run(stream)
     return output_combine
 
@@ -380,9 +386,7 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
-                          want_lse=False, stream_scratch=stream if q.is_cuda else None,
-                          counters=_stream_counters(q.device, stream) if kv_split > 0 else None,
-                          work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
     return call.run(stream)[0]
 
 
@@ -407,7 +411,7 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
     The reference runs a fixed grid of 132 programs that loop over (sequence, head, split) items and merge after a
     grid barrier on the int32 ``workspace``.  Here the same split count (32 unless ``kv_split`` says otherwise) runs
     as the work-queue form of the split kernel - two workgroups per compute unit pulling items - followed by the
-    combine kernel.  ``workspace`` is ignored: the reference's barrier works with any initial contents of it
+    combine kernel (``prepare_decode(..., single_launch=True)`` is the one-launch form; it is slower on MI355X).  ``workspace`` is ignored: the reference's barrier works with any initial contents of it
     (common_ops.py:57-81), whereas the queue's counters must be zero on entry, so the library always uses counters
     of its own (per stream, left at zero by every call).  The result is in q's dtype (the reference allocates
     float16 whatever q is)."""
@@ -416,7 +420,7 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap, kv_split=splits,
                           workspace=_as_scratch(output_split), out=output_combine, want_lse=False,
-                          stream_scratch=stream if q.is_cuda else None, counters=_stream_counters(q.device, stream))
+                          stream_scratch=stream if q.is_cuda else None)
     return call.run(stream)[0]
 
 
@@ -522,7 +526,7 @@ def flash_decode_bsnh(query: torch.Tensor, key_cache: torch.Tensor, value_cache:
     if query.is_cuda:
         stream = _stream_handle(stream)
     call = prepare_decode(query[:, 0], key_cache, value_cache, block_tables, kv_lens, sm_scale, soft_cap=soft_cap,
-                          out=output[:, 0], want_lse=False, work_queue=False)
+                          out=output[:, 0], want_lse=False, stream_scratch=stream, work_queue=False)
     call.run(stream)
     return output
 
