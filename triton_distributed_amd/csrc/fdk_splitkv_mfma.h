@@ -281,8 +281,28 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
     }
     const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
-    int first_pg = 0;
-    if (PM == PM_TILE) first_pg = tbl[min(c_start + tix * kTile, p.max_tokens - 1) >> p.page_shift];
+    const int pmask = p.page_size - 1;
+    struct PageIds { int32_t pg[PM == PM_TILE ? 1 : NJ]; };
+    // Page numbers of tile t, for any t: positions are clamped to the table only, not to the sequence, so that
+    // nothing here waits for kv_len.  The numbers of positions past the end are never used (a full tile has
+    // none; the partial last tile asks again, clamped to its last token).
+    auto pages_ahead = [&](int t, PageIds& pi) {
+        const int tok0 = c_start + t * kTile;
+        if (PM == PM_TILE) {
+            pi.pg[0] = tbl[min(tok0, p.max_tokens - 1) >> p.page_shift];
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                int n = tok0 + j * RPL;
+                if (PM >= PM_LANE) n += lrow;
+                n = min(n, p.max_tokens - 1);
+                pi.pg[PM == PM_TILE ? 0 : j] = tbl[PM == PM_LANE_DIV ? n / p.page_size : n >> p.page_shift];
+            }
+        }
+    };
+    PageIds pa, pb;                        // page numbers of the tiles that go to rg / rb
+    pages_ahead(tix, pa);
+    pages_ahead(tix + ti_n, pb);
     const int kv_len = min(p.kv_lens[b], p.max_tokens);
     if (c_start >= kv_len) {
         // kv_len == 0: a defined result where no combine follows (the first piece writes it)
@@ -302,16 +322,13 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     const char* kbase = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES + lpiece * 16;
     const char* vbase = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES + lpiece * 16;
-    const int pmask = p.page_size - 1;
     const uint32_t ksp_bytes = (uint32_t)(p.k_sp * ES), vsp_bytes = (uint32_t)(p.v_sp * ES);
     const uint32_t kst_bytes = (uint32_t)(p.k_st * ES), vst_bytes = (uint32_t)(p.v_st * ES);
     char* my_lds = lds + wave * kScratch;
     char* lds_k = my_lds;
     char* lds_v = my_lds + kScratch / 2;
 
-    struct PageIds { int32_t pg[PM == PM_TILE ? 1 : NJ]; };
-
-    auto pages_of = [&](int t, PageIds& pi) {
+    auto pages_of = [&](int t, PageIds& pi) {        // clamped to the sequence: for the partial last tile
         const int tok0 = c_start + t * kTile;
         if (PM == PM_TILE) {
             pi.pg[0] = tbl[min(tok0, c_end - 1) >> p.page_shift];      // clamped: any tile index may be asked for
@@ -325,11 +342,12 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             }
         }
     };
-    auto issue = [&](int t, const PageIds& pi, R& rg) {
+    auto issue = [&](int t, const PageIds& pi, R& rg, auto clamp_tag) {
         const int tok0 = c_start + t * kTile;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            const int n = min(tok0 + j * RPL + lrow, c_end - 1);      // clamp: always a valid, finite row
+            int n = tok0 + j * RPL + lrow;
+            if (decltype(clamp_tag)::value) n = min(n, c_end - 1);     // partial tile: always a valid, finite row
             const uint32_t slot = PM == PM_LANE_DIV ? n % p.page_size : (n & pmask);
             // page number x page stride: one 32 x 32 -> 64 bit multiply-add per address (the strides, in bytes, fit
             // 32 bits; a page number is never negative where it is used)
@@ -368,7 +386,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             for (int j = 0; j < NJ; ++j)
                 put(rg.v[j], load_stream16(kOffsetsInRegs ? vp + voff[j] : vp + j * vstep + voff[0]));
         } else {
-            issue(t, pi, rg);
+            issue(t, pi, rg, BoolTag<false>());
         }
     };
 
@@ -481,18 +499,13 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     const int n_full = (c_end - c_start) / kTile;
     {
         R rg;
-        PageIds pa, pb;                    // page numbers of the tiles that go to rg / rb
         int t = tix;
         const int st = ti_n;
-        if (t < n_full) {
-            if (PM == PM_TILE) pa.pg[0] = first_pg; else pages_of(t, pa);
-            pages_of(t + st, pb);
-            issue_full(t, pa, rg);
-        }
+        if (t < n_full) issue_full(t, pa, rg);
         if (NBUF == 1) {
             // one register buffer: the next tile's loads go into the registers just staged
             while (t < n_full) {
-                pages_of(t + 2 * st, pa);
+                pages_ahead(t + 2 * st, pa);
                 stage(rg);
                 const int tn = t + st;
                 if (tn < n_full) issue_full(tn, pb, rg);
@@ -505,11 +518,11 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             // always issues before it stages, so the waits on the older tile can be partial.
             R rb;
             while (t + 2 * st < n_full) {
-                pages_of(t + 2 * st, pa);
+                pages_ahead(t + 2 * st, pa);
                 issue_full(t + st, pb, rb);
                 stage(rg);
                 compute(t, BoolTag<false>());
-                pages_of(t + 3 * st, pb);
+                pages_ahead(t + 3 * st, pb);
                 issue_full(t + 2 * st, pa, rg);
                 stage(rb);
                 compute(t + st, BoolTag<false>());
@@ -528,7 +541,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         }
         if (n_full * kTile < c_end - c_start && (n_full % ti_n) == tix) {
             pages_of(n_full, pa);
-            issue(n_full, pa, rg);
+            issue(n_full, pa, rg, BoolTag<true>());
             stage(rg);
             compute(n_full, BoolTag<true>());
         }
