@@ -105,11 +105,13 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     // are never used) - the kernel is a chain of dependent memory round trips, this removes one or two.
     constexpr int kPre = 8;
     float pre[kPre][EPL];
+    float lse_early = 0.f;                       // chunk mode: lse of split `lane`, requested just as early
     if (!p.balanced) {
         const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
 #pragma unroll
         for (int j = 0; j < kPre; ++j)
             if (j < p.num_splits) Vec<EPL>::load(o_early + (int64_t)j * D, pre[j]);
+        if (lane < p.num_splits) lse_early = p.part_lse[row * p.num_splits + lane];
     }
     const PartRows pr = locate_rows<D>(p, b, h);
     const int live = pr.live;
@@ -127,7 +129,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
     for (int s0 = 0; s0 < live; s0 += 64) {
         const int n = min(64, live - s0);
-        const float my = lane < n ? lse_row[(s0 + lane) * pr.lse_step] * kLog2e : -INFINITY;   // log2 units
+        const float my = lane < n ? (!p.balanced && s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step]) * kLog2e
+                                  : -INFINITY;   // log2 units
         const float m_blk = wave_max(my);
         const float m_new = fmaxf(m_run, m_blk);
         const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
@@ -183,14 +186,17 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     const int wave = threadIdx.x >> 6;
     const int64_t row = blockIdx.x;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
-    // as in combine_kernel: the first kPre rows of this wavefront (s = wave, wave + 4, ...) are requested early
-    constexpr int kPre = 8;
+    // as in combine_kernel: the first kPre rows of this wavefront (s = wave, wave + 4, ...: all of them up to 64
+    // splits) and the lse values are requested before the number of live splits is known
+    constexpr int kPre = 16;
     float pre[kPre][EPL];
+    float lse_early = 0.f;
     if (!p.balanced) {
         const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
 #pragma unroll
         for (int j = 0; j < kPre; ++j)
             if (wave + kRowsPerWg * j < p.num_splits) Vec<EPL>::load(o_early + (int64_t)(wave + kRowsPerWg * j) * D, pre[j]);
+        if (lane < p.num_splits) lse_early = p.part_lse[row * p.num_splits + lane];
     }
     const PartRows pr = locate_rows<D>(p, b, h);
     const int live = pr.live;
@@ -205,7 +211,8 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     float m = -INFINITY;
     float my_first = -INFINITY;                    // lse of split `lane`, kept for the second pass
     for (int s0 = 0; s0 < live; s0 += 64) {
-        const float my = s0 + lane < live ? lse_row[(s0 + lane) * pr.lse_step] : -INFINITY;
+        const float my = s0 + lane < live ? (!p.balanced && s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step])
+                                          : -INFINITY;
         if (s0 == 0) my_first = my;
         m = fmaxf(m, wave_max(my));
     }

@@ -493,9 +493,12 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     // ---- pipeline over the full tiles: a tile is copied to LDS as soon as it has arrived, the next tile's
     // loads are issued into the same registers, and the arithmetic on the staged tile overlaps them.  The
     // partial last tile of the chunk goes to the wave whose turn it is.
-    // Page numbers run two tiles ahead of the arithmetic and are requested BEFORE the K/V loads of the tile in
-    // between: loads complete in order, so a page number requested after a tile's rows could only be used once
-    // those rows had arrived, and the tile after them could not be requested while they are under way.
+    // Page numbers run two tiles ahead of the arithmetic.  Per-lane page numbers (vector loads) are requested
+    // BEFORE the K/V loads of the tile in between: vector loads complete in order, so a page number requested
+    // after a tile's rows could only be used once those rows had arrived, and the tile after them could not be
+    // requested while they are under way.  Wave-uniform page numbers (scalar loads) are requested AFTER them:
+    // scalar loads complete in any order, so waiting for the older number also waits for the newest request.
+    constexpr bool kIdsFirst = PM >= PM_LANE;
     const int n_full = (c_end - c_start) / kTile;
     {
         R rg;
@@ -505,10 +508,11 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         if (NBUF == 1) {
             // one register buffer: the next tile's loads go into the registers just staged
             while (t < n_full) {
-                pages_ahead(t + 2 * st, pa);
+                if (kIdsFirst) pages_ahead(t + 2 * st, pa);
                 stage(rg);
                 const int tn = t + st;
                 if (tn < n_full) issue_full(tn, pb, rg);
+                if (!kIdsFirst) pages_ahead(t + 2 * st, pa);
                 compute(t, BoolTag<false>());
                 pb = pa;
                 t = tn;
@@ -518,12 +522,14 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             // always issues before it stages, so the waits on the older tile can be partial.
             R rb;
             while (t + 2 * st < n_full) {
-                pages_ahead(t + 2 * st, pa);
+                if (kIdsFirst) pages_ahead(t + 2 * st, pa);
                 issue_full(t + st, pb, rb);
+                if (!kIdsFirst) pages_ahead(t + 2 * st, pa);
                 stage(rg);
                 compute(t, BoolTag<false>());
-                pages_ahead(t + 3 * st, pb);
+                if (kIdsFirst) pages_ahead(t + 3 * st, pb);
                 issue_full(t + 2 * st, pa, rg);
+                if (!kIdsFirst) pages_ahead(t + 3 * st, pb);
                 stage(rb);
                 compute(t + st, BoolTag<false>());
                 t += 2 * st;
