@@ -16,6 +16,11 @@ namespace {
 
 constexpr int kRowsPerWg = 4;  // (b, h) rows per 256-thread workgroup
 
+// value of lane `i` (the same i in every lane) in all lanes
+__device__ __forceinline__ float bcast_lane(float x, int i) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), i));
+}
+
 // EPL adjacent fp32 values (EPL in {1, 2, 4}) with one load
 template <int EPL> struct Vec;
 template <> struct Vec<1> {
@@ -96,7 +101,7 @@ template <int D>
 __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     constexpr int EPL = D / 64;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + wave;   // b * Hq + h
     if (row >= (int64_t)p.batch * p.hq) return;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
 #pragma unroll
             for (int j = 0; j < kPre; ++j) {
                 if (j < n) {
-                    const float ws = __shfl(w, j, 64);
+                    const float ws = bcast_lane(w, j);
 #pragma unroll
                     for (int e = 0; e < EPL; ++e) acc[e] += ws * pre[j][e];
                 }
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
         }
 #pragma unroll 4
         for (; s < n; ++s) {
-            const float ws = __shfl(w, s, 64);
+            const float ws = bcast_lane(w, s);
             float o[EPL];
             Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
 #pragma unroll
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     constexpr int EPL = D / 64;
     __shared__ float sm[kRowsPerWg][D];
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t row = blockIdx.x;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
     // as in combine_kernel: the first kPre rows of this wavefront (s = wave, wave + 4, ...: all of them up to 64
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
 #pragma unroll
             for (int j = 0; j < kPre; ++j) {
                 if (wave + kRowsPerWg * j < n) {
-                    const float ws = __shfl(w, wave + kRowsPerWg * j, 64);
+                    const float ws = bcast_lane(w, wave + kRowsPerWg * j);
 #pragma unroll
                     for (int e = 0; e < EPL; ++e) acc[e] += ws * pre[j][e];
                 }
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
         }
 #pragma unroll 8
         for (; s < n; s += kRowsPerWg) {
-            const float ws = __shfl(w, s, 64);
+            const float ws = bcast_lane(w, s);
             float o[EPL];
             Vec<EPL>::load(o_row + (s0 + s) * pr.o_step, o);
 #pragma unroll
@@ -278,7 +283,7 @@ template <int D>
 __global__ __launch_bounds__(256) void combine_ranks_kernel(const CombineRanksParams p) {
     constexpr int EPL = D / 64;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + wave;
     if (row >= (int64_t)p.batch * p.hq) return;
     const int b = (int)(row / p.hq), h = (int)(row % p.hq);
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(256) void combine_ranks_kernel(const CombineRanksPa
 #pragma unroll
         for (int e = 0; e < EPL; ++e) acc[e] *= alpha;
         for (int s = 0; s < n; ++s) {
-            const float ws = __shfl(w, s, 64);
+            const float ws = bcast_lane(w, s);
             if (ws != 0.f) {   // wave-uniform; ranks without tokens may hold garbage rows
                 const int64_t base = (int64_t)(r0 + s) * p.stride_r + b * p.stride_b + h * p.stride_h + EPL * lane;
 #pragma unroll

@@ -177,15 +177,34 @@ __device__ __forceinline__ int wave_scan_i32(int x) {
 }
 __device__ __forceinline__ int wave_sum_i32(int x) { return __builtin_amdgcn_readlane(wave_scan_i32(x), 63); }
 
+// Reductions over the 64 lanes with DPP only (no LDS traffic): butterflies inside each row of 16, then the row
+// results are passed down the rows (row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3), so that
+// lane 63 holds the total, which every lane then reads.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_rows(float old, float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x),
+                                                                 CTRL, ROW_MASK, 0xF, false));
+}
+__device__ __forceinline__ float lane63(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
 __device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
-    return x;
+    x = fmaxf(x, dpp_mov<0xB1>(x));                 // quad_perm [1,0,3,2]   (permutations: every lane has a source)
+    x = fmaxf(x, dpp_mov<0x4E>(x));                 // quad_perm [2,3,0,1]
+    x = fmaxf(x, dpp_mov<0x141>(x));                // row_half_mirror
+    x = fmaxf(x, dpp_mov<0x140>(x));                // row_mirror
+    x = fmaxf(x, dpp_rows<0x142, 0xA>(x, x));       // rows that take no part keep their own value
+    x = fmaxf(x, dpp_rows<0x143, 0xC>(x, x));
+    return lane63(x);
 }
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o, 64);
-    return x;
+    x += dpp_mov<0xB1>(x);
+    x += dpp_mov<0x4E>(x);
+    x += dpp_mov<0x141>(x);
+    x += dpp_mov<0x140>(x);
+    x += dpp_rows<0x142, 0xA>(0.f, x);              // rows that take no part add nothing
+    x += dpp_rows<0x143, 0xC>(0.f, x);
+    return lane63(x);
 }
 
 // soft cap: cap * tanh(x / cap), tanh(y) = 1 - 2 / (exp(2y) + 1)
