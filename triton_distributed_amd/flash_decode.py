@@ -144,6 +144,37 @@ def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv
     return a
 
 
+_TEMPLATES = {}          # layout key -> (validated argument block without pointers, its plan)
+
+
+def _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len, k_scale, v_scale,
+                   algo, min_kv_len):
+    """``_fill_args`` + ``_plan_of`` with a cache: a serving loop calls with the same layouts over and over, and the
+    shape checks and the planning depend on shapes, strides, dtypes, devices and scalars only.  A hit copies the
+    validated block and sets the pointers (their alignment is checked by the library on every call)."""
+    def meta(t):
+        return None if t is None else (t.shape, t.stride(), t.dtype, t.device)
+    key = (meta(q), meta(k_cache), meta(v_cache), meta(block_table), meta(kv_lens), meta(k_scale), meta(v_scale),
+           sm_scale, soft_cap, kv_split, max_kv_len, min_kv_len, algo)
+    hit = _TEMPLATES.get(key)
+    if hit is None:
+        a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
+                       k_scale, v_scale, algo, min_kv_len=min_kv_len)
+        plan = _plan_of(a)
+        if len(_TEMPLATES) >= 256:
+            _TEMPLATES.clear()
+        _TEMPLATES[key] = (bytes(a), plan)
+        return a, plan
+    a = FdkDecodeArgs.from_buffer_copy(hit[0])
+    a.q, a.k_cache, a.v_cache = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr()
+    a.block_table, a.kv_lens = block_table.data_ptr(), kv_lens.data_ptr()
+    if k_scale is not None:
+        a.k_scale = k_scale.data_ptr()
+    if v_scale is not None:
+        a.v_scale = v_scale.data_ptr()
+    return a, hit[1]
+
+
 def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
     plan = FdkPlan()
     _lib.check(_LIB.fdk_plan(C.byref(a), num_cus, C.byref(plan)))
@@ -264,10 +295,9 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``run_static()``, which keeps the split partials in the library's own static scratch."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
-    a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
-                   k_scale, v_scale, algo, min_kv_len=min_kv_len)
+    a, plan = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
+                             k_scale, v_scale, algo, min_kv_len)
     batch, q_heads, d = q.shape
-    plan = _plan_of(a)
     if probe_loads:
         a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
