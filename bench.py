@@ -193,13 +193,16 @@ def bench_ceiling(args):
 
     dev = torch.device("cuda:0")
     inp = wl.make_inputs(args.config).to(dev)
-    if inp.cfg.kv_dtype == "fp8_e4m3" or inp.cfg.head_dim != 128:
-        print("--op ceiling: the load-pipeline probe is built for head_dim 128 and a 16-bit cache", file=sys.stderr)
+    if inp.cfg.head_dim != 128:
+        print("--op ceiling: the load-pipeline probe is built for head_dim 128", file=sys.stderr)
         sys.exit(2)
+    fp8 = inp.cfg.kv_dtype == "fp8_e4m3"
     alg_bytes = inp.algorithmic_bytes()
     g = torch.Generator(device=dev).manual_seed(inp.cfg.seed + 100)
-    pools = [(inp.k_cache, inp.v_cache),
-             tuple(torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype) for _ in range(2))]
+    mk = (lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
+        torch.float8_e4m3fn)) if fp8 else (lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev,
+                                                               dtype=inp.k_cache.dtype))
+    pools = [(inp.k_cache, inp.v_cache), (mk(), mk())]
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
               max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
     real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
@@ -208,7 +211,7 @@ def bench_ceiling(args):
     plan = real[0].plan
     single_pass = plan.num_splits == 1
     n_iter = args.steps
-    kv_bytes = sum(inp.kv_lens_host) * inp.cfg.kv_heads * 2 * inp.cfg.head_dim * 2
+    kv_bytes = sum(inp.kv_lens_host) * inp.cfg.kv_heads * 2 * inp.cfg.head_dim * (1 if fp8 else 2)
     lin_bytes = max(kv_bytes // 2 // 65536 * 65536, 1 << 20)       # per buffer: the K half, then the V half
     lin = [torch.randint(0, 255, (lin_bytes,), dtype=torch.uint8, device=dev) for _ in range(4)]
 

@@ -1247,3 +1247,23 @@ def test_single_launch_decode_against_the_oracle_and_the_two_launch_form(cuda_de
         assert torch.all(o1[dead] == 0) and torch.all(l1[dead] == float("-inf"))
     _check(o1[live], l1[live], q[live], k, v, table[live], [lens[b] for b in live], scale, ref_kv=ref_kv, tag=name)
     assert int(one._keep[-1].abs().sum()) == 0                  # the counters are back at zero
+
+
+def test_reference_entry_points_read_kv_split_as_an_upper_bound(cuda_device):
+    # the reference's layer passes kv_split = 32 for every shape (sp_flash_decode_layer.py:62)
+    import importlib
+    fd = importlib.import_module("triton_distributed_amd.flash_decode")
+    big = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=40, kv_len=600), cuda_device)
+    one = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=1, kv_len=16000), cuda_device)
+    args = lambda i: (i.q, i.k_cache, i.v_cache, i.block_table, i.kv_lens, i.sm_scale, 0.0)
+    assert fd._reference_kv_split(32, *args(big)) == -1          # 40 x 8 units fill the GPU: one pass, no chunks
+    assert fd._reference_kv_split(-1, *args(big)) == -1
+    own = tda.get_split_kv_plan(one.q, one.k_cache, one.v_cache, one.block_table, one.kv_lens)
+    assert own.num_splits > 4 and fd._reference_kv_split(4, *args(one)) == 4       # fewer than the library would take: forced
+    assert fd._reference_kv_split(1024, *args(one)) == -1
+    for inp in (big, one):
+        packed = tda.gqa_fwd_batch_decode_intra_rank(inp.q, inp.k_cache, inp.v_cache, None, None, inp.kv_lens,
+                                                     inp.block_table, inp.sm_scale, kv_split=32)
+        out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale, kv_split=32)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(packed[..., :128].float(), out.float(), atol=4e-3, rtol=2 ** -7)

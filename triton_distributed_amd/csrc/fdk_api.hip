@@ -335,8 +335,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
     sp.probe = (a->flags & FDK_FLAG_PROBE_LOADS) ? 1 : 0;
-    if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128 || a->kv_dtype == FDK_FP8_E4M3))
-        return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path, head_dim 128, 16-bit cache");
+    if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128))
+        return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path and head_dim 128");
     sp.scale_log2 = a->sm_scale * fdk::kLog2e;
     sp.soft_cap = a->soft_cap > 0.f ? a->soft_cap : 0.f;
     sp.sm_scale = a->sm_scale;

@@ -111,7 +111,7 @@ struct KvAppendParams {
 int launch_kv_append(const KvAppendParams& p, int qkv_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
-int launch_splitkv_mfma_probe(const SplitParams& p, hipStream_t stream);      // head_dim 128, 16-bit cache
+int launch_splitkv_mfma_probe(const SplitParams& p, int kv_dtype, hipStream_t stream);      // head_dim 128
 int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream);
 int launch_combine(const CombineParams& p, hipStream_t stream);
 int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);

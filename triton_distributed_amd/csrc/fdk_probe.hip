@@ -1,6 +1,6 @@
 // Measurement aids: what the memory system of this GPU delivers, with no arithmetic in the way.
 //   launch_splitkv_mfma_probe  the matrix-core split kernel reduced to its load pipeline (same pieces, same
-//                              addresses, same instructions in the same order) for head_dim 128 and a 16-bit cache
+//                              addresses, same instructions in the same order) for head_dim 128
 //   launch_linear_read         a plain streaming read of a buffer, with or without the non-temporal hint
 // Neither produces results; bench.py --op ceiling times them next to the real kernels.
 #include "fdk_splitkv_mfma.h"
@@ -46,9 +46,11 @@ __global__ __launch_bounds__(256) void linear_read_kernel(const u32x4_t* __restr
 
 }  // namespace
 
-int launch_splitkv_mfma_probe(const SplitParams& p, hipStream_t stream) {
+int launch_splitkv_mfma_probe(const SplitParams& p, int kv_dtype, hipStream_t stream) {
     if (p.head_dim != 128) return (int)hipErrorInvalidValue;
-    return launch_pm<FDK_BF16, false, 128, true>(p, stream);     // fp16 rows have the same bytes
+    // the q dtype does not matter to the loads: fp16 rows have the same bytes as bf16 rows
+    return kv_dtype == FDK_FP8_E4M3 ? launch_pm<FDK_BF16, true, 128, true>(p, stream)
+                                    : launch_pm<FDK_BF16, false, 128, true>(p, stream);
 }
 
 int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream) {

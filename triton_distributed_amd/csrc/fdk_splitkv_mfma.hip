@@ -39,7 +39,7 @@ int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg) {
 }
 
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
-    if (p.probe) return launch_splitkv_mfma_probe(p, stream);
+    if (p.probe) return launch_splitkv_mfma_probe(p, kv_dtype, stream);
     switch (p.head_dim) {
         case 64: return launch_splitkv_mfma_d64(p, q_dtype, kv_dtype, stream);
         case 128: return launch_splitkv_mfma_d128(p, q_dtype, kv_dtype, stream);

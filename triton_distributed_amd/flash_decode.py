@@ -24,7 +24,8 @@ current stream.  There is no fallback path: a missing library raises at import o
 
 Differences that a caller can observe
   * the split count defaults to a value chosen from the shape and the device's compute units
-    (reference: fixed 32, :863); ``kv_split`` still forces a count;
+    (reference: fixed 32, :863); ``kv_split`` forces a count in ``flash_decode`` / ``prepare_decode`` and is read as
+    an upper bound by the entry points that carry the reference's names (``_reference_kv_split``);
   * the per-split scratch is fp32 and private to the library: a caller-provided ``output_split`` is used
     as scratch only if it is large enough, its contents afterwards are unspecified;
   * ``workspace`` and ``q_lens`` are accepted and ignored, exactly as in the reference (:847, never read);
@@ -390,6 +391,22 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     return call.run(stream)
 
 
+def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap) -> int:
+    """How the drop-ins for the reference's entry points read ``kv_split`` (its ``NUM_KV_SPLITS``): as the most splits
+    to use, not as a count to force.  The reference's layer passes a fixed 32 (sp_flash_decode_layer.py:62) whatever the
+    shape; results do not depend on the count, and a batch that fills the GPU on its own is fastest with none (the
+    Llama-3-8B shape at batch 32: 87 us in one pass against 135 us in 32 chunks of 128 tokens).  If the plan the library
+    would choose on its own needs no more partial rows than ``kv_split`` allows it is used; otherwise the count is forced.
+    ``flash_decode`` / ``prepare_decode`` always force."""
+    if kv_split is None or kv_split <= 0:
+        return -1
+    if not isinstance(kv_lens, torch.Tensor) or not q.is_cuda:
+        return kv_split
+    # the same (cached) argument block and plan that the call itself uses when the library's own plan is taken
+    own = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, -1, None, None, None, "auto", None)[1]
+    return -1 if own.num_splits <= kv_split else kv_split
+
+
 def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
                                     soft_cap=0.0, output_split=None, output_combine=None, kv_split=-1,
                                     stream=None):
@@ -402,6 +419,7 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
         output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
     if q.is_cuda:
         stream = _stream_handle(stream)
+    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
                           want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
@@ -414,6 +432,7 @@ def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_
     """Drop-in for the reference function of the same name (flash_decode.py:763-844): ``[B, Hq, D]``."""
     if q.is_cuda:
         stream = _stream_handle(stream)
+    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
                           want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
@@ -445,7 +464,8 @@ def gqa_fwd_batch_decode_persistent(q, k_cache, v_cache, workspace, q_lens, kv_l
     (common_ops.py:57-81), whereas the queue's counters must be zero on entry, so the library always uses counters
     of its own (per stream, left at zero by every call).  The result is in q's dtype (the reference allocates
     float16 whatever q is)."""
-    splits = 32 if kv_split == -1 else kv_split
+    splits = _reference_kv_split(32 if kv_split == -1 else kv_split, q, k_cache, v_cache, block_table, kv_lens, scale,
+                                 soft_cap)
     if q.is_cuda:
         stream = _stream_handle(stream)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap, kv_split=splits,
