@@ -399,3 +399,33 @@ def test_kv_append_accepts_valid_arguments_and_rejects_bad_ones():
         rc = lib.fdk_kv_append(C.byref(_append_args(**{field: value})), None)
         assert rc == code, (field, value, rc, lib.fdk_last_error())
         assert lib.fdk_last_error() != b""
+
+
+def test_linear_read_probe_rejects_bad_arguments():
+    lib = _lib.load()
+    assert lib.fdk_probe_linear_read(None, 1 << 20, 1, 512, None) == _lib.FDK_ENULL
+    assert lib.fdk_probe_linear_read(0x10008, 1 << 20, 1, 512, None) == _lib.FDK_EALIGN
+    assert lib.fdk_probe_linear_read(0x10000, 1024, 1, 512, None) == _lib.FDK_ESHAPE
+    assert lib.fdk_probe_linear_read(0x10000, 1 << 20, 1, 0, None) == _lib.FDK_ESHAPE
+    assert lib.fdk_probe_linear_read(0x10000, 1 << 20, 1, 1 << 21, None) == _lib.FDK_ESHAPE
+
+
+def test_load_probe_flag_is_limited_to_what_is_built():
+    # the load-only variant of the split kernel exists for the matrix-core path and head_dim 128
+    ok = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS)
+    assert _decode_rc(ok) == 0
+    assert _decode_rc(_args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS, algo=_lib.FDK_ALGO_VALU)) == _lib.FDK_EUNSUPPORTED
+    wide = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS, head_dim=256, q_stride_b=32 * 256, q_stride_h=256,
+                 k_stride_page=16 * 8 * 256, k_stride_tok=8 * 256, k_stride_head=256, v_stride_page=16 * 8 * 256,
+                 v_stride_tok=8 * 256, v_stride_head=256, out_stride_b=32 * 256, out_stride_h=256)
+    assert _decode_rc(wide) == _lib.FDK_EUNSUPPORTED
+
+
+def test_single_launch_flag_needs_counters_to_take_effect():
+    # without counters the flag is ignored (split + combine); with them the usual checks on the counters apply
+    lib = _lib.load()
+    fl = _lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_SINGLE_LAUNCH
+    assert _decode_rc(_args(batch=4, flags=fl)) == 0
+    n = lib.fdk_counters_len(C.byref(_args(batch=4)))
+    assert _decode_rc(_args(batch=4, flags=fl, counters=0x90000, counters_len=n)) == 0
+    assert _decode_rc(_args(batch=4, flags=fl, counters=0x90000, counters_len=n - 1)) == _lib.FDK_EWORKSPACE

@@ -1267,3 +1267,24 @@ def test_reference_entry_points_read_kv_split_as_an_upper_bound(cuda_device):
         out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale, kv_split=32)
         torch.cuda.synchronize()
         torch.testing.assert_close(packed[..., :128].float(), out.float(), atol=4e-3, rtol=2 ** -7)
+
+
+def test_load_only_probes_run_and_leave_the_inputs_alone(cuda_device):
+    # measurement aids (bench.py --op ceiling): they produce no results, but must run on every plan mode and read only
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["ragged_g8"], batch=9, kv_len_range=(1, 9000)), cuda_device)
+    k0, v0, q0 = inp.k_cache.clone(), inp.v_cache.clone(), inp.q.clone()
+    for kw in (dict(), dict(kv_split=8), dict(kv_split=1)):
+        call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                  probe_loads=True, always_workspace=True, **kw)
+        call.run()
+        call.run_splitkv()
+    buf = torch.arange(1 << 22, dtype=torch.int32, device=cuda_device)
+    ref = buf.clone()
+    tda.probe_linear_read(buf, nontemporal=True)
+    tda.probe_linear_read(buf, nontemporal=False, workgroups=64)
+    torch.cuda.synchronize()
+    assert torch.equal(buf, ref) and torch.equal(inp.k_cache, k0) and torch.equal(inp.v_cache, v0) and torch.equal(inp.q, q0)
+    # the real call right after a probe call on the same buffers is unaffected
+    out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    torch.cuda.synchronize()
+    _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale, tag="after probe")
