@@ -664,7 +664,7 @@ def test_inter_rank_combine_equals_one_shot(cuda_device):
 
 # ---- large batches: single pass with blocks of 4 or 8 kv heads per (eight-wave) workgroup ------------------------------
 @pytest.mark.parametrize("heads,batch,want_nh", [((32, 8), 256, 8), ((32, 8), 128, 4), ((16, 4), 256, 4), ((48, 2), 300, 2),
-                                                ((8, 8), 300, 8), ((96, 4), 130, 4)])
+                                                ((8, 8), 300, 8), ((96, 4), 130, 4), ((32, 8), 32, 1), ((24, 3), 100, 1)])
 @pytest.mark.parametrize("d,dtype,fp8,page", [(128, torch.bfloat16, False, 16), (128, torch.float16, False, 1),
                                              (128, torch.bfloat16, True, 16), (64, torch.bfloat16, False, 6),
                                              (256, torch.float16, False, 16), (256, torch.bfloat16, True, 64)])
@@ -703,6 +703,55 @@ def test_large_batches_take_wide_head_blocks(cuda_device, heads, batch, want_nh,
            tag=f"wide blocks nh={want_nh}")
     # the same call with the head block forced apart (a split count forces chunk mode with narrower blocks)
     out2, lse2 = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, kv_split=2)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    torch.testing.assert_close(out[live].float(), out2[live].float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse[live], lse2[live], atol=1e-4, rtol=0)
+
+
+# ---- single pass with one kv head per workgroup: the split kernel runs with one register buffer per wavefront ----------
+@pytest.mark.parametrize("d,dtype,fp8,page", [(128, torch.bfloat16, False, 16), (128, torch.float16, False, 1),
+                                             (128, torch.bfloat16, False, 8), (128, torch.bfloat16, False, 6),
+                                             (128, torch.float16, True, 16), (128, torch.bfloat16, True, 1),
+                                             (64, torch.bfloat16, False, 16), (64, torch.float16, True, 3)])
+def test_single_pass_with_one_kv_head_per_workgroup(cuda_device, d, dtype, fp8, page):
+    """Batch 32 x 8 kv heads gives exactly one workgroup per compute unit of a 256-unit GPU, each on one kv head: the
+    plan of the headline configuration.  Lengths from 0 to 1500 tokens (up to 24 tiles per wavefront), every page mode."""
+    batch, hq, hkv = 32, 32, 8
+    print(f"case one head per workgroup D={d} {dtype} fp8={fp8} P={page}", flush=True)
+    g = torch.Generator().manual_seed(d + page + (7 if fp8 else 0))
+    lens = torch.randint(1, 1501, (batch,), generator=g).tolist()
+    lens[0], lens[1], lens[2], lens[3], lens[batch - 1] = 1500, 0, 1, 16, 17
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 2
+    q = torch.randn(batch, hq, d, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, max(pages) + 1), -7, dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t)
+    from triton_distributed_amd import _lib
+    if _lib.load().fdk_device_cus() == 256:
+        assert plan.num_splits == 1 and plan.kv_heads_per_wg == 1, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    assert (out[1] == 0).all() and (lse[1] == float("-inf")).all()
+    rows = [0, 2, 3, 4, 9, 17, 30, batch - 1]
+    _check(out[rows], lse[rows], q[rows], k, v, table[rows], [lens[i] for i in rows], d ** -0.5, ref_kv=ref_kv,
+           tag="one head per workgroup")
+    # the same call cut into chunks (two register buffers, partial rows, combine launch)
+    out2, lse2 = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, kv_split=3)
     torch.cuda.synchronize()
     live = [i for i, n in enumerate(lens) if n > 0]
     torch.testing.assert_close(out[live].float(), out2[live].float(), atol=1e-2, rtol=1e-2)

@@ -443,11 +443,27 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         constexpr bool MASKED = decltype(masked_tag)::value;
         const int tok0 = c_start + t * kTile;
         // ---- S^T[token][head] = K Q^T ----
+        // All LDS reads of the tile are requested up front (K rows, then the transposed V blocks, which do not
+        // depend on the softmax): a wavefront is alone on its SIMD in the single-pass plans, so a read that is
+        // requested only when its MFMA is due costs its full latency every time (worth 0.5-1 % on 16-bit caches).
         f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+        uint4 ka[KS];
+        // Not for the widest rows (no registers to spare) nor for fp8 caches (two wavefronts per SIMD already
+        // overlap, and the longer register lifetimes cost more than they gain: measured 1 % slower).
+        constexpr bool kReadVEarly = D <= 128 && !FP8;
+        const int k4 = c >> 2, cc = c & 3;
+        const int vrow = 4 * a + k4;
+        uint2 va[DB];
+        if (kReadVEarly) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) ka[ks] = *reinterpret_cast<const uint4*>(lds_k + k_off<RB>(c, 4 * ks + a));
+#pragma unroll
+            for (int db = 0; db < DB; ++db) va[db] = M::read_tr(lds_v + v_off<RB>(vrow, 2 * db + (cc >> 1)) + (cc & 1) * 8);
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const uint4 ka = *reinterpret_cast<const uint4*>(lds_k + k_off<RB>(c, 4 * ks + a));
-            s = M::qk(ka, qb[ks], s);
+            if (!kReadVEarly) ka[ks] = *reinterpret_cast<const uint4*>(lds_k + k_off<RB>(c, 4 * ks + a));
+            s = M::qk(ka[ks], qb[ks], s);
         }
         // ---- online softmax for head c over tokens 4a .. 4a+3 of this tile ----
         float sv[4] = {s.x, s.y, s.z, s.w};
@@ -481,12 +497,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         // reference does before its second dot (flash_decode.py:230)
         const uint2 pb = make_uint2(P2::pack(pr[0], pr[1]), P2::pack(pr[2], pr[3]));
         // ---- O^T[d][head] += V^T P^T ----
-        const int k4 = c >> 2, cc = c & 3;
-        const int vrow = 4 * a + k4;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            const uint2 va = M::read_tr(lds_v + v_off<RB>(vrow, 2 * db + (cc >> 1)) + (cc & 1) * 8);
-            acc[db] = M::pv(va, pb, acc[db]);
+            if (!kReadVEarly) va[db] = M::read_tr(lds_v + v_off<RB>(vrow, 2 * db + (cc >> 1)) + (cc & 1) * 8);
+            acc[db] = M::pv(va[db], pb, acc[db]);
         }
     };
 
@@ -853,17 +867,29 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     p.persistent = (p.counters != nullptr && !p.direct && !p.balanced && p.total_items > resident) ? 1 : 0;
     const dim3 grid((unsigned)(p.balanced ? p.workgroups : p.persistent ? resident : p.total_items));
     const dim3 block(64 * nw);
-    // Two register buffers per wavefront, except for the widest rows where they would not leave room for two
-    // workgroups per compute unit.
-    constexpr int NBUF = D > 128 ? 1 : 2;
-#define FDK_MFMA_LAUNCH(PMV) \
-    hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NBUF, D, PROBE>), grid, block, lds_bytes, stream, p)
-    switch (pm) {
-        case PM_TILE: FDK_MFMA_LAUNCH(PM_TILE); break;
-        case PM_LOAD: FDK_MFMA_LAUNCH(PM_LOAD); break;
-        case PM_LANE: FDK_MFMA_LAUNCH(PM_LANE); break;
-        default: FDK_MFMA_LAUNCH(PM_LANE_DIV); break;
+    // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on).  Two by
+    // default.  One for the widest rows (two would not leave room for two workgroups per compute unit), and one
+    // where a single pass gives every compute unit one workgroup whose four wavefronts share ONE kv head: a
+    // wavefront then keeps exactly one tile under way, 32 KB per compute unit, which is what the memory system
+    // needs to stay busy; a second tile only queues up and the pass takes 3-4 % longer at every length
+    // (batch 32 x 8 kv heads, 512 ... 32768 tokens).  Plans with several heads per workgroup or two workgroups
+    // per compute unit measure the same or up to 1 % better with two.
+    const bool one_buffer = D > 128 || (p.hg_per_wg == 1 && p.num_splits == 1 && !p.balanced);
+#define FDK_MFMA_LAUNCH(PMV, NB) \
+    hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
+#define FDK_MFMA_LAUNCH_PM(NB)                                    \
+    switch (pm) {                                                 \
+        case PM_TILE: FDK_MFMA_LAUNCH(PM_TILE, NB); break;        \
+        case PM_LOAD: FDK_MFMA_LAUNCH(PM_LOAD, NB); break;        \
+        case PM_LANE: FDK_MFMA_LAUNCH(PM_LANE, NB); break;        \
+        default: FDK_MFMA_LAUNCH(PM_LANE_DIV, NB); break;         \
     }
+    if (one_buffer) {
+        FDK_MFMA_LAUNCH_PM(1)
+    } else {
+        FDK_MFMA_LAUNCH_PM((D > 128 ? 1 : 2))
+    }
+#undef FDK_MFMA_LAUNCH_PM
 #undef FDK_MFMA_LAUNCH
     return (int)hipGetLastError();
 }
