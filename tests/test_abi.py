@@ -167,8 +167,10 @@ def test_static_scratch_entry_validates_like_fdk_decode():
 
 
 def test_workspace_is_required_only_when_the_plan_splits():
-    # 32 sequences x 8 kv heads fill 256 compute units on their own: one pass, no scratch
-    assert _decode_rc(_args(workspace=None, workspace_bytes=0)) == 0
+    # 32 sequences x 8 kv heads, all known to be 4096 tokens long, fill 256 compute units on their own: one pass,
+    # no scratch.  Without the lower bound the lengths may differ: equal shares, partial rows, scratch.
+    assert _decode_rc(_args(workspace=None, workspace_bytes=0, max_kv_len=4096, min_kv_len=4096)) == 0
+    assert _decode_rc(_args(workspace=None, workspace_bytes=0)) == _lib.FDK_EWORKSPACE
     # 4 sequences do not: the KV range is split and the partials need scratch
     assert _decode_rc(_args(batch=4, workspace=None)) == _lib.FDK_EWORKSPACE
     assert _decode_rc(_args(batch=4, workspace_bytes=1024)) == _lib.FDK_EWORKSPACE
@@ -233,9 +235,24 @@ def _plan(a, cus=256):
 
 
 def test_plan_scales_splits_with_occupancy():
-    p = _plan(_args())                                    # 256 (sequence, kv head) units on 256 CUs
+    p = _plan(_args(max_kv_len=4096, min_kv_len=4096))    # 256 (sequence, kv head) units of equal length on 256 CUs
     assert p.num_splits == 1 and p.chunk_tokens >= 4096   # they fill the device: one pass, no combine
-    assert p.algo == _lib.FDK_ALGO_MFMA
+    assert p.algo == _lib.FDK_ALGO_MFMA and p.kv_heads_per_wg == 1
+    # the same batch with lengths the host does not vouch for: a single pass would be as slow as its longest
+    # sequence, so the tokens are cut into equal shares (two workgroups per compute unit, two kv heads each)
+    p = _plan(_args())
+    assert p.balanced == 1 and p.workgroups == 512 and p.kv_heads_per_wg == 2 and p.num_splits > 1
+    assert _plan(_args(max_kv_len=4096, min_kv_len=2000)).balanced == 1
+    # short contexts keep the single pass (nothing to gain from cutting them), and so do batches with four or more
+    # workgroups per compute unit, which even out by themselves
+    assert _plan(_args(max_kv_len=1024)).num_splits == 1
+    p = _plan(_args(batch=1024, q_stride_b=32 * 128, out_stride_b=32 * 128))
+    assert p.num_splits == 1 and p.balanced == 0 and p.kv_heads_per_wg == 8
+    # equal lengths that fill the compute units unevenly (40 x 8 units on 256: a quarter of them carry two) are
+    # cut into equal shares as well; 60 x 8 fill them well enough
+    assert _plan(_args(batch=40, max_kv_len=4096, min_kv_len=4096)).balanced == 1
+    p = _plan(_args(batch=60, max_kv_len=4096, min_kv_len=4096))
+    assert p.balanced == 0 and p.num_splits == 1
     # fewer sequences, short context: chunk mode - chunks are multiples of 64 tokens and cover the range
     p4 = _plan(_args(batch=4))
     assert p4.balanced == 0 and p4.num_splits > 1 and p4.chunk_tokens % 64 == 0

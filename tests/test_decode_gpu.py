@@ -1184,6 +1184,23 @@ def test_config2_llama3_8b_b32(cuda_device, algo):
     _check_rows(inp, out, lse, range(32) if algo == "auto" else range(0, 32, 5), "cfg2")
 
 
+def _hinted_single_pass(cuda_device, name, rows):
+    # bench.py passes the host-known length bounds: equal bounds say that the sequences are alike, which is what a
+    # single pass (whole sequences per workgroup, no partial rows, no combine launch) needs; without them the same
+    # configuration runs as equal shares
+    cfg = wl.CONFIGS[name]
+    hints = dict(max_kv_len=cfg.kv_len, min_kv_len=cfg.kv_len)
+    inp, out, lse = _full_config(name, cuda_device, **hints)
+    plan = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, **hints)
+    assert not plan.balanced and plan.num_splits == 1
+    assert tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens).balanced
+    _check_rows(inp, out, lse, rows, f"{name} hinted")
+
+
+def test_config2_llama3_8b_b32_with_the_length_hints_of_the_benchmark(cuda_device):
+    _hinted_single_pass(cuda_device, "llama3_8b_b32", range(0, 32, 3))
+
+
 @pytest.mark.parametrize("algo", ["auto", "valu"])
 def test_config3_ragged_g8(cuda_device, algo):
     inp, out, lse = _full_config("ragged_g8", cuda_device, algo)
@@ -1200,6 +1217,10 @@ def test_config4_long_131k(cuda_device, algo):
 def test_config5_fp8_70b_b128(cuda_device, algo):
     inp, out, lse = _full_config("fp8_70b_b128", cuda_device, algo)
     _check_rows(inp, out, lse, range(0, 128, 9) if algo == "auto" else [5, 100], "cfg5")
+
+
+def test_config5_fp8_70b_b128_with_the_length_hints_of_the_benchmark(cuda_device):
+    _hinted_single_pass(cuda_device, "fp8_70b_b128", range(0, 128, 11))
 
 
 def test_config4_long_131k_with_the_length_hints_of_the_benchmark(cuda_device):

@@ -69,6 +69,10 @@ constexpr int64_t kMaxTableTokens = (int64_t)1 << 30;
 constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and never asks the runtime
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
+constexpr int kMinRaggedLen = 2048;      // shorter contexts: a single pass that fills the compute units stays
+constexpr int64_t kPieceOverheadBytes = 72 << 10;   // balanced mode: see piece_cost_granules
+constexpr double kStreamBytesPerUs = 6.5e6;   // what a well-filled split kernel streams (plan estimates only)
+constexpr double kSplitOverheadUs = 7.0;      // partial rows + combine launch of a split plan (plan estimates only)
 
 // Scratch of fdk_decode_static: one copy per GPU, part of the loaded code object, never allocated or freed.
 constexpr size_t kStaticScratchBytes = FDK_STATIC_SCRATCH_BYTES;
@@ -209,6 +213,36 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         units_per_seq = fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
     }
     const int64_t units = (int64_t)batch * units_per_seq;
+    const int single_pass_heads_per_wg = kv_heads_per_wg;
+
+    // A single pass gives every workgroup whole sequences, which is only as good as the sequences are alike and
+    // as evenly as the workgroups fill the compute units.  It is replaced by balanced mode (equal shares of the
+    // tokens that kv_lens holds, narrow head blocks, a combine launch) when
+    //  - the host has not said that the lengths are alike (min_kv_len) and there are fewer than four workgroups
+    //    per compute unit to even things out (batch 64 x 8 kv heads, lengths uniform in [1, 8192]: 223 us as a
+    //    single pass, the longest sequence decides) and the sequences can be long (max_len >= kMinRaggedLen); or
+    //  - the lengths are alike but the workgroups do not fill the compute units evenly - 1.25 per compute unit:
+    //    a quarter of the compute units carry two and finish long after the rest - and the estimate says that
+    //    pays for the combine launch.  Measured for batch 40 / 48 / 60 x 8 kv heads x 4096 tokens: the single
+    //    pass runs at (fill + 1) / 2 of the even rate, fill = units / (rounds x compute units): 131 / 139 /
+    //    159 us against 103 / 124 / 155 us of streaming time.
+    const bool alike = a->min_kv_len > 0 && (int64_t)a->min_kv_len * 32 >= max_len * 31;
+    bool rebalance = false;
+    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && units >= num_cus && batch <= kMaxBalancedBatch) {
+        if (!alike) {
+            rebalance = units < 4 * (int64_t)num_cus && max_len >= kMinRaggedLen;
+        } else if (units > num_cus) {
+            const int64_t rounds = cdiv64(units, num_cus);
+            const double fill = (double)units / (double)(rounds * num_cus);
+            const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * 2.0 * a->head_dim *
+                                     elem_size(a->kv_dtype) / kStreamBytesPerUs;
+            rebalance = stream_us * 2.0 / (fill + 1.0) > 1.05 * (stream_us * 1.03 + kSplitOverheadUs);
+        }
+        if (rebalance) {
+            kv_heads_per_wg = a->num_kv_heads % 2 ? 1 : 2;
+            units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg);
+        }
+    }
 
     // Split count: none when the (sequence, head block) units alone fill the compute units - a single pass
     // then writes the final result and no combine runs.  Otherwise the per-sequence chunks aim at one workgroup
@@ -221,11 +255,11 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     if (min_chunk < kMinChunk) min_chunk = kMinChunk;
     if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
     const int64_t most_chunks = cdiv64(max_len, min_chunk);
-    const bool may_split = a->num_splits <= 0 && units < num_cus && most_chunks > 1;
+    const bool may_split = a->num_splits <= 0 && (units < num_cus || rebalance) && most_chunks > 1;
     int64_t splits = 1;
     if (a->num_splits > 0) {
         splits = a->num_splits;
-    } else if (may_split) {
+    } else if (may_split && !rebalance) {
         splits = (int64_t)num_cus / units;
         if (splits > most_chunks) splits = most_chunks;
     }
@@ -239,7 +273,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // needs none of that: per-sequence chunks, one workgroup per compute unit, are 2-7 % faster there.  The workspace then holds (shares + batch) slots of
     // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
     const int64_t columns = (int64_t)batch * cdiv64(max_len, fdk::kBalanceGranule);   // granules of all sequences, at most
-    const bool uniform = a->min_kv_len > 0 && (int64_t)a->min_kv_len * 32 >= max_len * 31;
+    const bool uniform = alike && !rebalance;
     if (algo == FDK_ALGO_MFMA && may_split && !uniform && batch <= kMaxBalancedBatch &&
         columns < (1 << 30)) {                                            // the kernel counts granules in int32
         const int64_t gran = fdk::kBalanceGranule;
@@ -260,6 +294,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
             return FDK_OK;
         }
     }
+    if (rebalance) plan->kv_heads_per_wg = single_pass_heads_per_wg;     // no equal shares after all: the single pass
     int64_t chunk = cdiv64(cdiv64(max_len, splits), kChunkAlign) * kChunkAlign;
     if (a->num_splits <= 0) splits = cdiv64(max_len, chunk);   // drop splits that would always be empty
     if (splits > kMaxSplits) {
@@ -269,6 +304,15 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     plan->num_splits = (int32_t)splits;
     plan->chunk_tokens = (int32_t)chunk;
     return FDK_OK;
+}
+
+// Balanced mode: what starting one more sequence costs a workgroup, in granules of the partition.  The fixed
+// time of a piece (table and q loads before its first rows, the merge of the wavefronts after its last) is
+// what a workgroup needs to stream about kPieceOverheadBytes.
+int piece_cost_granules(const fdk_decode_args* a, int kv_heads_per_wg) {
+    const int64_t granule_bytes = (int64_t)fdk::kBalanceGranule * kv_heads_per_wg * 2 * a->head_dim * elem_size(a->kv_dtype);
+    const int64_t c = (kPieceOverheadBytes + granule_bytes / 2) / granule_bytes;
+    return (int)(c > 16 ? 16 : c);
 }
 
 // q-head tiles per kv head, as the resolved algorithm's kernel counts them
@@ -331,6 +375,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.workgroups = r->plan.workgroups;
     sp.heads_per_tile = sp.group < 16 ? sp.group : 16;
     sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
+    sp.piece_cost = sp.balanced ? piece_cost_granules(a, sp.hg_per_wg) : 0;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
@@ -354,6 +399,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     cp.group = sp.group; cp.kv_heads_per_wg = sp.hg_per_wg; cp.head_tiles = sp.head_tiles;
     cp.hg_blocks = a->num_kv_heads / (sp.hg_per_wg > 0 ? sp.hg_per_wg : 1);
     cp.rows_per_slot = sp.rows_per_slot; cp.heads_per_tile = sp.heads_per_tile;
+    cp.piece_cost = sp.piece_cost;
     return FDK_OK;
 }
 

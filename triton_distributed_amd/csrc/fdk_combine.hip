@@ -67,15 +67,17 @@ __device__ __forceinline__ PartRows locate_rows(const CombineParams& p, int b, i
     // [before, before + mine); the piece of share wc for unit u is in slot (wc + b) * units + u.
     const int lane = threadIdx.x & 63;
     const int units = p.hg_blocks * p.head_tiles;
+    // (a sequence with tokens counts for p.piece_cost granules more, in front of its own: see the split kernel)
     int total = 0, before = 0;
     for (int b0 = 0; b0 < p.batch; b0 += 64) {
         const int bb = b0 + lane;
-        const int g = bb < p.batch ? (max(min(p.kv_lens[bb], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule : 0;
+        int g = bb < p.batch ? (max(min(p.kv_lens[bb], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule : 0;
+        if (g > 0) g += p.piece_cost;
         total += g;
         before += bb < b ? g : 0;
     }
     total = wave_sum_i32(total);
-    before = wave_sum_i32(before);
+    before = wave_sum_i32(before) + p.piece_cost;          // where the granules of sequence b begin
     const int mine = (max(min(p.kv_lens[b], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule;
     const int kvh = h / p.group, hin = h % p.group;
     const int u = (kvh / p.kv_heads_per_wg) * p.head_tiles + hin / 16;

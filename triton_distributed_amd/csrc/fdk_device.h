@@ -45,6 +45,7 @@ struct SplitParams {
     int32_t persistent, total_items, num_cus;
     int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
+    int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
     int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its
@@ -68,7 +69,7 @@ struct CombineParams {
     int32_t pack_lse;
     // balanced mode (see the split kernel): where the pieces of a (sequence, head) row are
     int32_t balanced, workgroups;
-    int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile;
+    int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile, piece_cost;
 };
 
 struct CombineRanksParams {

@@ -590,7 +590,9 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     }
     if (ti_n > 1) __syncthreads();                           // ti_n == 1: a wave reads back only its own rows
     if (live) {
-        constexpr int kMaxShare = 4;                         // at most four wavefronts share a kv head
+        // wavefronts that share a kv head, at most: eight where tiles are small (see launch_pm), else four (the
+        // wider merge costs a short piece 0.8 us)
+        constexpr int kMaxShare = 2 * kTile * D * (FP8 ? 1 : 2) <= 4096 ? 8 : 4;
         float mw[kMaxShare], lw[kMaxShare];
         float mx = -INFINITY;
 #pragma unroll
@@ -714,7 +716,14 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         return;
     }
     const int units = p.hg_blocks * p.head_tiles;
-    auto granules_of = [&](int bb) { return (max(min(p.kv_lens[bb], p.max_tokens), 0) + kGranule - 1) / kGranule; };
+    // A sequence counts for its granules plus p.piece_cost more in front of them (none if it is empty): every
+    // sequence a share begins costs its workgroup a fixed time (table and q loads before the first rows, the merge
+    // of the wavefronts after the last), and a share that starts several sequences gets fewer tokens for it.
+    const int pc = p.piece_cost;
+    auto granules_of = [&](int bb) {
+        const int g = (max(min(p.kv_lens[bb], p.max_tokens), 0) + kGranule - 1) / kGranule;
+        return g > 0 ? g + pc : 0;
+    };
     int item = blockIdx.x;                        // chunk mode: current item
     int x = 0, hi = 0;                            // balanced mode: next granule, end of this workgroup's share
     int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
@@ -771,8 +780,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             pb = b;
             hgb = bu / p.head_tiles;
             ht = bu % p.head_tiles;
-            c_start = (x - before) * kGranule;
-            c_limit = (piece_end - before) * kGranule;
+            c_start = max(x - before - pc, 0) * kGranule;                // the first pc positions hold no tokens
+            c_limit = (piece_end - before - pc) * kGranule;              // <= 0: nothing of this sequence in the share
             const int64_t slot = (int64_t)(wc + b) * units + bu;
             prow0 = slot * p.rows_per_slot + hl * p.heads_per_tile;
             prow_step = 1;
@@ -782,7 +791,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                 const int big = share_r * (share_q + 1);
                 return g < big ? g / (share_q + 1) : share_r + (g - big) / share_q;
             };
-            const int wc_first = share_of(before);
+            const int wc_first = share_of(before + pc);
             mr.live = share_of(before + gb - 1) - wc_first + 1;
             mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
             mr.piece_step = (int64_t)units * p.rows_per_slot;
@@ -815,7 +824,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         prow_step = __builtin_amdgcn_readfirstlane(prow_step);
         prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(prow0 >> 32)) << 32) |
                 (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)prow0);
-        run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step, mr);
+        if (!p.balanced || c_limit > 0) run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step, mr);
         if (p.balanced) {
             x = piece_end;
             if (x >= hi) return;
@@ -852,7 +861,19 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     p.head_tiles = (p.group + 15) / 16;
     if (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) p.hg_per_wg = 1;
     p.hg_blocks = p.hkv / p.hg_per_wg;
-    const int nw = p.hg_per_wg >= 4 ? 8 : 4;      // wavefronts per workgroup (see mfma_kv_heads_per_wg)
+    // How much a compute unit keeps under way decides how well the memory system runs, and about 32 KB is the
+    // optimum on MI355X (a tile of 16 tokens is kTileBytes per wavefront): less leaves it idle, more only queues
+    // up and costs 3-5 %.  A single pass (one workgroup per compute unit) is shaped for that: wavefronts per
+    // workgroup and register buffers per wavefront (below) follow from the tile size; blocks of 4 or 8 kv heads
+    // always take 8 wavefronts.  Measured, batch 32 x 8 kv heads x 4096 tokens: 16-bit cache 85.3 us with two
+    // buffers, 81.7 us with one; fp8 cache 52.3 us with 4 wavefronts x 2 buffers, 47.1 us with 8 x 1.
+    constexpr int kTileBytes = 2 * kTile * D * (FP8 ? 1 : 2);                    // K and V rows of one tile
+    const int64_t items = (int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles;
+    const bool single_pass = p.num_splits == 1 && !p.balanced;
+    // small tiles: also per-sequence chunks that give each compute unit at most one workgroup (one-byte-per-value
+    // caches cut like that measure 13-16 % faster with 8 wavefronts x 1 buffer than with 4 x 2)
+    const bool shaped = single_pass || (kTileBytes <= 4096 && !p.balanced && items <= (p.num_cus > 0 ? p.num_cus : 256));
+    const int nw = (p.hg_per_wg >= 4 || (shaped && kTileBytes <= 4096)) ? 8 : 4;      // wavefronts per workgroup
     const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float)) + 16;
     constexpr int RPL = Regs<FP8, D>::RPL;
     int pm;
@@ -867,14 +888,11 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     p.persistent = (p.counters != nullptr && !p.direct && !p.balanced && p.total_items > resident) ? 1 : 0;
     const dim3 grid((unsigned)(p.balanced ? p.workgroups : p.persistent ? resident : p.total_items));
     const dim3 block(64 * nw);
-    // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on).  Two by
-    // default.  One for the widest rows (two would not leave room for two workgroups per compute unit), and one
-    // where a single pass gives every compute unit one workgroup whose four wavefronts share ONE kv head: a
-    // wavefront then keeps exactly one tile under way, 32 KB per compute unit, which is what the memory system
-    // needs to stay busy; a second tile only queues up and the pass takes 3-4 % longer at every length
-    // (batch 32 x 8 kv heads, 512 ... 32768 tokens).  Plans with several heads per workgroup or two workgroups
-    // per compute unit measure the same or up to 1 % better with two.
-    const bool one_buffer = D > 128 || (p.hg_per_wg == 1 && p.num_splits == 1 && !p.balanced);
+    // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on): two, or
+    // one for the widest rows (two would not leave room for two workgroups per compute unit) and in a single
+    // pass whose wavefronts together hold 32 KB with one.  Plans that split the KV range (two workgroups per
+    // compute unit, short pieces) measure the same or up to 1 % better with two.
+    const bool one_buffer = D > 128 || (shaped && kTileBytes * nw >= 32768);
 #define FDK_MFMA_LAUNCH(PMV, NB) \
     hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
 #define FDK_MFMA_LAUNCH_PM(NB)                                    \
