@@ -41,6 +41,7 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
 enum PageMode { PM_TILE = 0, PM_LOAD = 1, PM_LANE = 2, PM_LANE_DIV = 3 };
 template <bool B> struct BoolTag { static constexpr bool value = B; };
+template <int N> struct IntTag { static constexpr int value = N; };
 
 constexpr int kTile = 16;                 // tokens per tile
 constexpr int kGranule = kBalanceGranule; // balanced mode: tokens per unit of the partition
@@ -590,60 +591,62 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     }
     if (ti_n > 1) __syncthreads();                           // ti_n == 1: a wave reads back only its own rows
     if (live) {
-        // wavefronts that share a kv head, at most: eight where tiles are small (see launch_pm), else four (the
-        // wider merge costs a short piece 0.8 us)
-        constexpr int kMaxShare = 2 * kTile * D * (FP8 ? 1 : 2) <= 4096 ? 8 : 4;
-        float mw[kMaxShare], lw[kMaxShare];
-        float mx = -INFINITY;
+        // The merge is written out for each number of wavefronts that share a kv head (1, 2, 4; 8 where tiles
+        // are small, see launch_pm): straight-line code keeps all LDS reads of a column block under way together.
+        const int hq = head0 + c;
+        float lse_nat = 0.f;
+        auto merge = [&](auto share_tag) {
+            constexpr int TI = decltype(share_tag)::value;
+            float mw[TI], lw[TI];
+            float mx = -INFINITY;
 #pragma unroll
-        for (int t = 0; t < kMaxShare; ++t) {
-            mw[t] = -INFINITY;
-            lw[t] = 0.f;
-            if (t < ti_n) {
+            for (int t = 0; t < TI; ++t) {
                 mw[t] = sm_m[(hl + nh * t) * 16 + c];
                 lw[t] = sm_l[(hl + nh * t) * 16 + c];
+                mx = fmaxf(mx, mw[t]);
             }
-            mx = fmaxf(mx, mw[t]);
-        }
-        float sc[kMaxShare], l = 0.f;
+            float sc[TI], l = 0.f;
 #pragma unroll
-        for (int t = 0; t < kMaxShare; ++t) {
-            sc[t] = fast_exp2(mw[t] - mx);                   // mx is finite: the chunk holds >= 1 token
-            l += lw[t] * sc[t];
-        }
-        const float norm = vscale * fast_rcp(l);
-        const int hq = head0 + c;
-        const float lse_nat = (mx + fast_log2(l)) * kLn2;
-        for (int db = tix; db < DB; db += ti_n) {
-            float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int t = 0; t < TI; ++t) {
+                sc[t] = fast_exp2(mw[t] - mx);                   // mx is finite: the chunk holds >= 1 token
+                l += lw[t] * sc[t];
+            }
+            const float norm = vscale * fast_rcp(l);
+            lse_nat = (mx + fast_log2(l)) * kLn2;
 #pragma unroll
-            for (int t = 0; t < kMaxShare; ++t) {
-                if (t < ti_n) {
-                    const float4 x = reinterpret_cast<const float4*>(lds + (hl + nh * t) * kScratch)[db * 64 + lane];
-                    o.x += x.x * sc[t];
-                    o.y += x.y * sc[t];
-                    o.z += x.z * sc[t];
-                    o.w += x.w * sc[t];
+            for (int t = 0; t < TI; ++t) sc[t] *= norm;
+            for (int db = tix; db < DB; db += TI) {
+                float4 x[TI];
+#pragma unroll
+                for (int t = 0; t < TI; ++t) x[t] = reinterpret_cast<const float4*>(lds + (hl + nh * t) * kScratch)[db * 64 + lane];
+                float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int t = 0; t < TI; ++t) {
+                    o.x += x[t].x * sc[t];
+                    o.y += x[t].y * sc[t];
+                    o.z += x[t].z * sc[t];
+                    o.w += x[t].w * sc[t];
                 }
-            }
-            o.x *= norm;
-            o.y *= norm;
-            o.z *= norm;
-            o.w *= norm;
-            const int d0 = 16 * db + 4 * a;
-            if (p.direct) {
-                const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0;
-                store_out4(p.out, ob, o, p.out_dtype);
-            } else {
-                float* dst = p.part_o + (prow0 + (int64_t)c * prow_step) * D + d0;
-                if (p.fused) {
-                    st_agent2(dst, o.x, o.y);
-                    st_agent2(dst + 2, o.z, o.w);
+                const int d0 = 16 * db + 4 * a;
+                if (p.direct) {
+                    const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0;
+                    store_out4(p.out, ob, o, p.out_dtype);
                 } else {
-                    *reinterpret_cast<float4*>(dst) = o;
+                    float* dst = p.part_o + (prow0 + (int64_t)c * prow_step) * D + d0;
+                    if (p.fused) {
+                        st_agent2(dst, o.x, o.y);
+                        st_agent2(dst + 2, o.z, o.w);
+                    } else {
+                        *reinterpret_cast<float4*>(dst) = o;
+                    }
                 }
             }
-        }
+        };
+        constexpr bool kSmallTiles = 2 * kTile * D * (FP8 ? 1 : 2) <= 4096;
+        if (ti_n == 1) merge(IntTag<1>());
+        else if (ti_n == 2) merge(IntTag<2>());
+        else if (ti_n == 4 || !kSmallTiles) merge(IntTag<4>());
+        else merge(IntTag<kSmallTiles ? 8 : 4>());
         if (tix == 0 && a == 0) {
             if (p.direct) {
                 if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
@@ -791,12 +794,15 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                 const int big = share_r * (share_q + 1);
                 return g < big ? g / (share_q + 1) : share_r + (g - big) / share_q;
             };
-            const int wc_first = share_of(before + pc);
-            mr.live = share_of(before + gb - 1) - wc_first + 1;
-            mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
-            mr.piece_step = (int64_t)units * p.rows_per_slot;
-            mr.hl_step = p.heads_per_tile;
-            mr.g_step = 1;
+            mr = MergeRows{0, 0, 0, 0, 0};
+            if (p.fused) {                       // (two integer divisions each: not on the way to the first loads)
+                const int wc_first = share_of(before + pc);
+                mr.live = share_of(before + gb - 1) - wc_first + 1;
+                mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
+                mr.piece_step = (int64_t)units * p.rows_per_slot;
+                mr.hl_step = p.heads_per_tile;
+                mr.g_step = 1;
+            }
         } else {
             int wg = item;
             ht = wg % p.head_tiles;
