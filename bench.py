@@ -32,13 +32,25 @@ def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=-1,
+                    help="untimed warm-up steps (default: at least 100 and at least 0.3 s of calls - the GPU clock needs some "
+                         "tens of milliseconds of load to come up after the idle time of the input generation, which "
+                         "kernels with much arithmetic per byte (fp8 cache) feel)")
     ap.add_argument("--config", default="llama3_8b_b32")
     ap.add_argument("--rotate", type=int, default=2,
                     help="distinct KV pools cycled through, so the working set exceeds the 256 MB memory-side cache "
                          "(raised automatically until the pools together exceed 1 GB)")
     ap.add_argument("--kv-split", type=int, default=-1)
     ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
+    ap.add_argument("--wavefronts", type=int, default=0, choices=[0, 4, 8],
+                    help="measurement aid: wavefronts per workgroup of the matrix-core split kernel (0: the library's choice)")
+    ap.add_argument("--buffers", type=int, default=0, choices=[0, 1, 2],
+                    help="measurement aid: register buffers (tiles of loads under way) per wavefront (0: the library's choice)")
+    ap.add_argument("--no-hints", action="store_true",
+                    help="do not pass the host-known length bounds (max_kv_len / min_kv_len): the plan of a caller that "
+                         "knows nothing about the lengths")
+    ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size")
+    ap.add_argument("--kv-len", type=int, default=0, help="override the configuration's (uniform) kv_len")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
     ap.add_argument("--single-launch", action="store_true",
@@ -139,6 +151,8 @@ def bench_kv_append(args):
     def step():
         tda.qk_norm_rope_update_kvcache(qkv, k, v, table, lens, wq, wk, cos, sin, q_out, k_scale=ks, v_scale=ks)
 
+    if args.warmup < 0:
+        args.warmup = 100
     for _ in range(args.warmup):
         step()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -192,7 +206,7 @@ def bench_ceiling(args):
     from triton_distributed_amd import workloads as wl
 
     dev = torch.device("cuda:0")
-    inp = wl.make_inputs(args.config).to(dev)
+    inp = wl.make_inputs(_config_of(args, wl)).to(dev)
     if inp.cfg.head_dim != 128:
         print("--op ceiling: the load-pipeline probe is built for head_dim 128", file=sys.stderr)
         sys.exit(2)
@@ -204,7 +218,7 @@ def bench_ceiling(args):
                                                                dtype=inp.k_cache.dtype))
     pools = [(inp.k_cache, inp.v_cache), (mk(), mk())]
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
-              max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+              wavefronts=args.wavefronts, buffers=args.buffers, **_hints_of(args, inp))
     real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
     probe = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, probe_loads=True, **kw)
              for k, v in pools]
@@ -249,6 +263,29 @@ def bench_ceiling(args):
     }), flush=True)
 
 
+def _config_of(args, wl):
+    """The named configuration, with --batch / --kv-len applied."""
+    cfg = wl.CONFIGS[args.config]
+    if args.batch > 0 or args.kv_len > 0:
+        import dataclasses
+        kw = {}
+        if args.batch > 0:
+            kw["batch"] = args.batch
+        if args.kv_len > 0:
+            if cfg.kv_len is None:
+                kw["kv_len_range"] = (cfg.kv_len_range[0], args.kv_len)
+            else:
+                kw["kv_len"] = args.kv_len
+        cfg = dataclasses.replace(cfg, **kw, description=cfg.description + " [" + ", ".join(
+            f"{k} = {v}" for k, v in kw.items()) + "]")
+    return cfg
+
+
+def _hints_of(args, inp):
+    """Host-known length bounds for the planner (none with --no-hints)."""
+    return {} if args.no_hints else dict(max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -270,7 +307,7 @@ def main():
     if args.op == "ceiling":
         return bench_ceiling(args)
     t_gen = time.perf_counter()
-    inp_cpu = wl.make_inputs(args.config)
+    inp_cpu = wl.make_inputs(_config_of(args, wl))
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
     inp = inp_cpu.to(dev)
     pools = [(inp.k_cache, inp.v_cache)]
@@ -289,8 +326,8 @@ def main():
         pools.append((mk(), mk()))
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
-                                max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host),
-                                single_launch=args.single_launch)
+                                single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
+                                **_hints_of(args, inp))
              for k, v in pools]
     plan = calls[0].plan
     alg_bytes = inp.algorithmic_bytes()
@@ -313,6 +350,16 @@ def main():
         calls[i % len(calls)].run()
 
     # ---- whole call: W warm-up, then exactly K timed steps ----------------------------------------------------
+    if args.warmup < 0:
+        for i in range(10):
+            step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(20):
+            step(i)
+        torch.cuda.synchronize()
+        per_call = max((time.perf_counter() - t0) / 20, 1e-6)
+        args.warmup = max(100, int(0.3 / per_call))
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -368,8 +415,7 @@ def main():
         graph_us = (time.perf_counter() - t0) * 1e6 / (reps * len(calls))
 
     # ---- the un-prepared public entry point: flash_decode() validates, marshals and allocates (out, lse) per call
-    kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo,
-              max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
+    kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, **_hints_of(args, inp))
     n_entry = min(args.steps, 100)
     for i in range(5):
         tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens, inp.sm_scale, **kw)
@@ -383,7 +429,8 @@ def main():
     traffic = None
     traffic_source = None
     tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
+    resized = args.batch > 0 or args.kv_len > 0
+    if os.path.exists(tpath) and not resized and not args.kv_split > 0 and not args.no_hints:
         with open(tpath) as f:
             traffic = json.load(f).get(args.config, {}).get("bytes_per_launch")
         if traffic is not None:
@@ -392,7 +439,8 @@ def main():
     qd = inp.cfg.q_dtype
     result = {
         "metric": "decode-attn achieved HBM GB/s (algorithmic bytes / time per call; µs/call alongside), "
-                  "Llama-3-8B shape b=32" if args.config == "llama3_8b_b32" else f"decode-attn achieved HBM GB/s, {args.config}",
+                  "Llama-3-8B shape b=32" if args.config == "llama3_8b_b32" and not resized else
+                  f"decode-attn achieved HBM GB/s, {inp.cfg.name}" + (" (resized)" if resized else ""),
         "value": round(gbps, 1),
         "unit": "GB/s",
         "us_per_call": round(ms_per_step * 1e3, 2),
@@ -417,7 +465,8 @@ def main():
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "single_launch": bool(args.single_launch and plan.num_splits > 1),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
-            "host_length_hints": [min(inp.kv_lens_host), max(inp.kv_lens_host)],
+            "host_length_hints": None if args.no_hints else [min(inp.kv_lens_host), max(inp.kv_lens_host)],
+            "wavefronts_override": args.wavefronts or None, "buffers_override": args.buffers or None,
         },
         "roofline": {
             "bound": "hbm",

@@ -40,7 +40,7 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
          offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
-         offsetof(fdk_decode_args, counters_len));
+         offsetof(fdk_decode_args, tune_buffers));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
@@ -57,7 +57,7 @@ int main(void) {
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
                                        ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
-                                        "counters_len")]
+                                        "tune_buffers")]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -210,6 +210,17 @@ def test_dry_run_refuses_what_a_real_call_would_refuse():
     assert lib.fdk_decode_splitkv(C.byref(a), None) == _lib.FDK_ESHAPE
     # a misaligned workspace
     assert _decode_rc(_args(batch=4, workspace=0x80004)) == _lib.FDK_EALIGN
+
+
+def test_tuning_overrides_are_validated():
+    # measurement aids: 0 (the library's choice), 4 or 8 wavefronts, 1 or 2 buffers; anything else is refused
+    for wf, nb, rc in [(0, 0, 0), (4, 1, 0), (8, 2, 0), (8, 0, 0), (2, 0, _lib.FDK_ESHAPE), (16, 0, _lib.FDK_ESHAPE),
+                       (0, 3, _lib.FDK_ESHAPE), (0, -1, _lib.FDK_ESHAPE)]:
+        assert _decode_rc(_args(tune_wavefronts=wf, tune_buffers=nb)) == rc, (wf, nb)
+    # they never change the plan
+    p0, p1 = _plan(_args()), _plan(_args(tune_wavefronts=8, tune_buffers=1))
+    assert (p0.num_splits, p0.balanced, p0.workgroups, p0.kv_heads_per_wg) == (p1.num_splits, p1.balanced, p1.workgroups,
+                                                                                p1.kv_heads_per_wg)
 
 
 def test_packed_output_needs_a_wider_row():

@@ -758,6 +758,50 @@ def test_single_pass_with_one_kv_head_per_workgroup(cuda_device, d, dtype, fp8, 
     torch.testing.assert_close(lse[live], lse2[live], atol=1e-4, rtol=0)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("hints", [True, False])
+def test_kernel_shape_overrides_change_timing_only(cuda_device, fp8, hints):
+    """wavefronts / buffers (measurement aids) select how the split kernel is shaped; every combination the kernel
+    accepts gives the result of the library's own choice (same arithmetic per wavefront: bit-identical with the same
+    number of wavefronts, within rounding otherwise), and combinations it cannot run are ignored."""
+    batch, hq, hkv, d, page = 32, 32, 8, 128, 16
+    g = torch.Generator().manual_seed(77)
+    lens = [2100] * batch if hints else torch.randint(1, 2101, (batch,), generator=g).tolist()
+    lens[0] = 2100
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 1
+    q = torch.randn(batch, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.zeros((batch, max(pages)), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table, lens_t = table.to(cuda_device), _lens_t(lens, cuda_device)
+    ks = vs = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+    kw = dict(k_scale=ks, v_scale=vs, max_kv_len=max(lens))
+    if hints:
+        kw["min_kv_len"] = min(lens)             # alike lengths: a single pass; without: equal shares
+    base = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, **kw)
+    assert base.plan.balanced == (not hints)
+    out0, lse0 = (t.clone() for t in base.run())
+    torch.cuda.synchronize()
+    for wf in (0, 4, 8):
+        for nb in (0, 1, 2):
+            print(f"case overrides fp8={fp8} hints={hints} wavefronts={wf} buffers={nb}", flush=True)
+            out, lse = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, wavefronts=wf, buffers=nb, **kw).run()
+            torch.cuda.synchronize()
+            torch.testing.assert_close(out.float(), out0.float(), atol=1e-2, rtol=1e-2)
+            torch.testing.assert_close(lse, lse0, atol=1e-5, rtol=0)
+    with pytest.raises(Exception):
+        tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, wavefronts=3, **kw).run()
+
+
 # ---- balanced mode: the kernel cuts the batch's KV ranges into equal shares from kv_lens ---------------------------
 BALANCED_CASES = {
     # name: (kv_lens, (Hq, Hkv), page, head_dim, fp8)

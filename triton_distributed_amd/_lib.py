@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 6
+FDK_ABI_VERSION = 7
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -54,6 +54,7 @@ class FdkDecodeArgs(C.Structure):
         ("lse", C.c_void_p), ("lse_stride_b", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("counters", C.c_void_p), ("counters_len", C.c_int64),
+        ("tune_wavefronts", C.c_int32), ("tune_buffers", C.c_int32),
     ]
 
 

@@ -128,6 +128,9 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if (a->kv_dtype != a->q_dtype && a->kv_dtype != FDK_FP8_E4M3)
         return fail(FDK_EUNSUPPORTED, "kv_dtype %d must equal q_dtype or be fp8_e4m3", a->kv_dtype);
     if (a->algo < FDK_ALGO_AUTO || a->algo > FDK_ALGO_MFMA) return fail(FDK_EUNSUPPORTED, "algo %d", a->algo);
+    if ((a->tune_wavefronts != 0 && a->tune_wavefronts != 4 && a->tune_wavefronts != 8) ||
+        (a->tune_buffers < 0 || a->tune_buffers > 2))
+        return fail(FDK_ESHAPE, "tune_wavefronts %d (0, 4, 8) / tune_buffers %d (0, 1, 2)", a->tune_wavefronts, a->tune_buffers);
     if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
     if (!(a->soft_cap <= FLT_MAX)) return fail(FDK_ESHAPE, "soft_cap is not a finite number (<= 0 switches it off)");
     if (a->batch == 0) return FDK_OK;
@@ -376,6 +379,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.heads_per_tile = sp.group < 16 ? sp.group : 16;
     sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
     sp.piece_cost = sp.balanced ? piece_cost_granules(a, sp.hg_per_wg) : 0;
+    sp.tune_wavefronts = a->tune_wavefronts;
+    sp.tune_buffers = a->tune_buffers;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;

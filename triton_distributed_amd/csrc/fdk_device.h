@@ -46,6 +46,7 @@ struct SplitParams {
     int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
+    int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
     int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its

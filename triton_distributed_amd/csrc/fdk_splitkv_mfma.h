@@ -879,7 +879,11 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // small tiles: also per-sequence chunks that give each compute unit at most one workgroup (one-byte-per-value
     // caches cut like that measure 13-16 % faster with 8 wavefronts x 1 buffer than with 4 x 2)
     const bool shaped = single_pass || (kTileBytes <= 4096 && !p.balanced && items <= (p.num_cus > 0 ? p.num_cus : 256));
-    const int nw = (p.hg_per_wg >= 4 || (shaped && kTileBytes <= 4096)) ? 8 : 4;      // wavefronts per workgroup
+    int nw = (p.hg_per_wg >= 4 || (shaped && kTileBytes <= 4096)) ? 8 : 4;            // wavefronts per workgroup
+    // a caller's override (measurements), if the kernel can run it: every kv head of the block needs a wavefront,
+    // and at most four (small tiles: eight) wavefronts share a head
+    if (p.tune_wavefronts >= p.hg_per_wg && p.tune_wavefronts / p.hg_per_wg <= (kTileBytes <= 4096 ? 8 : 4))
+        nw = p.tune_wavefronts;
     const size_t lds_bytes = (size_t)nw * (kScratch + 2 * 16 * sizeof(float)) + 16;
     constexpr int RPL = Regs<FP8, D>::RPL;
     int pm;
@@ -898,7 +902,7 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // one for the widest rows (two would not leave room for two workgroups per compute unit) and in a single
     // pass whose wavefronts together hold 32 KB with one.  Plans that split the KV range (two workgroups per
     // compute unit, short pieces) measure the same or up to 1 % better with two.
-    const bool one_buffer = D > 128 || (shaped && kTileBytes * nw >= 32768);
+    const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1 : (shaped && kTileBytes * nw >= 32768));
 #define FDK_MFMA_LAUNCH(PMV, NB) \
     hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
 #define FDK_MFMA_LAUNCH_PM(NB)                                    \

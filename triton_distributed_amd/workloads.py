@@ -48,6 +48,13 @@ CONFIGS: Dict[str, DecodeConfig] = {
 }
 CONFIG_ORDER: List[str] = ["tiny", "llama3_8b_b32", "ragged_g8", "long_131k", "fp8_70b_b128"]
 
+# Two more shapes for the measurements behind the plan choices (not benchmark configurations): a ragged batch whose
+# (sequence, kv head) units would fill the GPU as a single pass, and the headline shape with an fp8 cache.
+CONFIGS["ragged_b64_8kv"] = DecodeConfig("ragged_b64_8kv", 1201, 64, 32, 8, 128, 16, kv_len_range=(1, 8192),
+                                         description="B64 32q/8kv D128 N~U[1,8192] P16 bf16")
+CONFIGS["fp8_8b_b32"] = DecodeConfig("fp8_8b_b32", 1202, 32, 32, 8, 128, 16, kv_len=4096, kv_dtype="fp8_e4m3",
+                                     description="B32 32q/8kv D128 N4096 P16, e4m3 KV with per-kv-head scales")
+
 # The shape behind the reference's only published figure for this path (README.md:200-202; perf loops of
 # test/nvidia/test_sp_decode_attn.py:203-220 and test_decode_attn.py:294-527): batch 1, 96 q / 12 kv heads,
 # head_dim 128, fp16, page size 1, local KV 8K ... 128K.
