@@ -33,7 +33,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=-1,
-                    help="untimed warm-up steps (default: at least 100 and at least 0.3 s of calls - the GPU clock needs some "
+                    help="untimed warm-up steps (default: at least 100 and at least 0.1 s of calls - the GPU clock needs some "
                          "tens of milliseconds of load to come up after the idle time of the input generation, which "
                          "kernels with much arithmetic per byte (fp8 cache) feel)")
     ap.add_argument("--config", default="llama3_8b_b32")
@@ -359,7 +359,7 @@ def main():
             step(i)
         torch.cuda.synchronize()
         per_call = max((time.perf_counter() - t0) / 20, 1e-6)
-        args.warmup = max(100, int(0.3 / per_call))
+        args.warmup = max(100, int(0.1 / per_call))
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()

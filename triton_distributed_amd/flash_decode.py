@@ -379,7 +379,9 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     max_kv_len   host-known upper bound of kv_lens, used only to size the splits
                  (default ``max_pages * P``)
     min_kv_len   host-known lower bound of kv_lens (default: unknown).  A batch whose bounds lie within 1/32 of
-                 each other is cut into per-sequence chunks instead of balanced shares; results never depend on it
+                 each other gets whole sequences per workgroup (a single pass where they fill the GPU, else
+                 per-sequence chunks); otherwise long contexts are cut into equal shares of the tokens on the
+                 device (a single pass is as slow as its longest sequence); results never depend on it
     k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
