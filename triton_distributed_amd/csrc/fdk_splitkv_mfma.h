@@ -38,6 +38,8 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+typedef const __attribute__((address_space(4))) int32_t* ConstI32;     // read-only for the whole kernel
+__device__ __forceinline__ ConstI32 as_const(const int32_t* p) { return (ConstI32)(uintptr_t)p; }
 
 enum PageMode { PM_TILE = 0, PM_LOAD = 1, PM_LANE = 2, PM_LANE_DIV = 3 };
 template <bool B> struct BoolTag { static constexpr bool value = B; };
@@ -281,7 +283,12 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qb[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
     }
-    const int32_t* tbl = p.block_table + (int64_t)b * p.tbl_sb;
+    // block_table and kv_lens are never written by this kernel: read through the constant address space, so that
+    // wave-uniform reads stay scalar loads on every code path.  (Where a piece follows another in a loop, the
+    // compiler otherwise assumes that the previous piece's stores may have changed them and falls back to vector
+    // loads, which complete in order with the K/V loads: waiting for a page number then waits for the tile of rows
+    // requested before it, and the loop of an fp8 cache ran 20 % slower.)
+    const ConstI32 tbl = as_const(p.block_table + (int64_t)b * p.tbl_sb);
     const int pmask = p.page_size - 1;
     struct PageIds { int32_t pg[PM == PM_TILE ? 1 : NJ]; };
     // Page numbers of tile t, for any t: positions are clamped to the table only, not to the sequence, so that
@@ -304,7 +311,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     PageIds pa, pb;                        // page numbers of the tiles that go to rg / rb
     pages_ahead(tix, pa);
     pages_ahead(tix + ti_n, pb);
-    const int kv_len = min(p.kv_lens[b], p.max_tokens);
+    const int kv_len = min(as_const(p.kv_lens)[b], p.max_tokens);
     if (c_start >= kv_len) {
         // kv_len == 0: a defined result where no combine follows (the first piece writes it)
         if ((p.direct || (p.fused && c_start == 0)) && tix == 0) write_empty_rows(b, head0, heads_here);
@@ -315,8 +322,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
 
     float kscale = 1.f, vscale = 1.f;
     if (FP8) {
-        if (p.k_scale) kscale = p.k_scale[kvh];
-        if (p.v_scale) vscale = p.v_scale[kvh];
+        if (p.k_scale) kscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.k_scale))[kvh]);
+        if (p.v_scale) vscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.v_scale))[kvh]);
     }
     const bool softcap = p.soft_cap > 0.f;
     const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
@@ -724,7 +731,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     // of the wavefronts after the last), and a share that starts several sequences gets fewer tokens for it.
     const int pc = p.piece_cost;
     auto granules_of = [&](int bb) {
-        const int g = (max(min(p.kv_lens[bb], p.max_tokens), 0) + kGranule - 1) / kGranule;
+        const int g = (max(min(as_const(p.kv_lens)[bb], p.max_tokens), 0) + kGranule - 1) / kGranule;
         return g > 0 ? g + pc : 0;
     };
     int item = blockIdx.x;                        // chunk mode: current item

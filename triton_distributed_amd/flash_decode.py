@@ -399,9 +399,10 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
 def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap) -> int:
     """How the drop-ins for the reference's entry points read ``kv_split`` (its ``NUM_KV_SPLITS``): as the most splits
     to use, not as a count to force.  The reference's layer passes a fixed 32 (sp_flash_decode_layer.py:62) whatever the
-    shape; results do not depend on the count, and a batch that fills the GPU on its own is fastest with none (the
-    Llama-3-8B shape at batch 32: 87 us in one pass against 135 us in 32 chunks of 128 tokens).  If the plan the library
-    would choose on its own needs no more partial rows than ``kv_split`` allows it is used; otherwise the count is forced.
+    shape; results do not depend on the count, and a batch that fills the GPU on its own is not to be cut into 32 chunks
+    per sequence (the Llama-3-8B shape at batch 32: 89 us as equal shares of the tokens, 135 us in 32 chunks of 128
+    tokens).  If the plan the library would choose on its own needs no more partial rows than ``kv_split`` allows it is
+    used; otherwise the count is forced.
     ``flash_decode`` / ``prepare_decode`` always force."""
     if kv_split is None or kv_split <= 0:
         return -1
