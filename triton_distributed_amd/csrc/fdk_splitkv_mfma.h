@@ -906,10 +906,13 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     const dim3 grid((unsigned)(p.balanced ? p.workgroups : p.persistent ? resident : p.total_items));
     const dim3 block(64 * nw);
     // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on): two, or
-    // one for the widest rows (two would not leave room for two workgroups per compute unit) and in a single
-    // pass whose wavefronts together hold 32 KB with one.  Plans that split the KV range (two workgroups per
-    // compute unit, short pieces) measure the same or up to 1 % better with two.
-    const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1 : (shaped && kTileBytes * nw >= 32768));
+    // one for the widest rows (two would not leave room for two workgroups per compute unit), in a single pass
+    // whose wavefronts together hold 32 KB with one, and for long pieces with wave-uniform page numbers (two
+    // workgroups per compute unit already hold 64 KB with one: 0.6-1.4 % faster).  Short pieces, and page sizes
+    // whose page numbers come by vector loads (in order with the rows), are up to 7 % faster with two.
+    const bool long_pieces = pm == PM_TILE && !single_pass && p.chunk >= 512;
+    const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1
+                                                       : ((shaped && kTileBytes * nw >= 32768) || long_pieces));
 #define FDK_MFMA_LAUNCH(PMV, NB) \
     hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
 #define FDK_MFMA_LAUNCH_PM(NB)                                    \
