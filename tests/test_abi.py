@@ -270,6 +270,13 @@ def test_plan_scales_splits_with_occupancy():
     assert p4.num_splits * p4.chunk_tokens >= 4096 > (p4.num_splits - 1) * p4.chunk_tokens
     # chunk mode aims at one workgroup per compute unit and never launches more than there are compute units
     assert p4.kv_heads_per_wg == 2 and p4.num_splits == 256 // (4 * 4)
+    # chunks end on tile boundaries (16 tokens), not coarser: 6 head blocks x 42 chunks of 208 tokens use 252 of the
+    # 256 compute units for the reference's benchmark shape at 8K (rounded to 64 tokens it would be 32 x 256 on 192)
+    p_ref = _plan(_args(batch=1, num_q_heads=96, num_kv_heads=12, page_size=1, max_pages=8192, table_stride_b=8192,
+                        k_stride_page=12 * 128, k_stride_tok=12 * 128, v_stride_page=12 * 128, v_stride_tok=12 * 128,
+                        q_stride_b=96 * 128, out_stride_b=96 * 128, lse_stride_b=96))
+    assert p_ref.balanced == 0 and p_ref.chunk_tokens % 16 == 0 and p_ref.kv_heads_per_wg == 2
+    assert 6 * p_ref.num_splits <= 256 < 6 * (p_ref.num_splits + 3)
     p24 = _plan(_args(batch=24, max_pages=64, table_stride_b=64))       # 96 units, 1024 tokens
     assert p24.balanced == 0 and p24.num_splits == 2 and p24.chunk_tokens == 512
     # few units, long context: balanced mode - two workgroups per compute unit share the KV ranges of the whole
