@@ -342,8 +342,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     const int S = r->plan.num_splits;
     const bool direct = direct_ok && S == 1;
     const int64_t rows = (int64_t)a->batch * a->num_q_heads;
-    if ((int64_t)a->batch * S * a->num_kv_heads * head_tiles_of(a, r->plan.algo) > INT32_MAX)
-        return fail(FDK_ESHAPE, "grid too large");
+    if ((int64_t)a->batch * S * a->num_kv_heads * head_tiles_of(a, r->plan.algo) > INT32_MAX || a->batch > 65535)
+        return fail(FDK_ESHAPE, "grid too large (batch x splits x heads; at most 65535 sequences)");
     float* part_o = nullptr;
     float* part_lse = nullptr;
     if (!direct && a->batch > 0) {

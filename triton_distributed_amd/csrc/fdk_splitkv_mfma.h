@@ -701,8 +701,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     // counters[1] counts finished workgroups, and the last one to finish puts both back to zero.  The first item
     // of every workgroup is its own index.
     // Balanced mode: the sequences, counted in granules of kGranule tokens and laid end to end, are cut into
-    // gridDim.x / units equal shares (fewer if there are fewer granules), units = (kv-head block, q-head tile)
-    // pairs of a sequence; workgroup (share wc, unit u) = blockIdx.x works its share off for its unit, sequence
+    // gridDim.y equal shares (fewer if there are fewer granules), units = (kv-head block, q-head tile)
+    // pairs of a sequence; workgroup (share wc, unit u) = (blockIdx.y, blockIdx.x) works its share off for its unit, sequence
     // by sequence.  Its partial rows for sequence b go to slot (wc + b) * units + u: pieces are ordered by
     // (wc, b) with at least one of the two growing from one piece to the next, so the slot is unique, and the
     // pieces of a sequence occupy consecutive wc.  Neighbouring workgroups read the same tokens of neighbouring
@@ -710,14 +710,15 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     if (!p.balanced && !p.persistent) {
         // The common chunk-mode case is kept free of the loop below: straight-line code lets the compiler
         // overlap the first loads of the piece (about a microsecond per workgroup on MI355X).
-        int wg = blockIdx.x;
-        if (wg >= p.total_items) return;
-        const int ht = wg % p.head_tiles;
-        wg /= p.head_tiles;
-        const int hgb = wg % p.hg_blocks;
-        wg /= p.hg_blocks;
-        const int split = wg % p.num_splits;
-        const int pb = wg / p.num_splits;
+        // grid = (head blocks x head tiles, splits, sequences): the piece follows from the block index without a
+        // division, so the table and q loads of the piece can be requested as soon as the arguments are there.
+        // (Workgroups are handed out in x-major order: neighbours still read neighbouring heads of the same tokens.)
+        const int split = blockIdx.y, pb = blockIdx.z;
+        int ht = 0, hgb = blockIdx.x;
+        if (p.head_tiles > 1) {
+            ht = blockIdx.x % p.head_tiles;
+            hgb = blockIdx.x / p.head_tiles;
+        }
         // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
         const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
         run_piece(pb, hgb, ht, split * p.chunk, split == p.num_splits - 1 ? p.max_tokens : split * p.chunk + p.chunk,
@@ -737,14 +738,14 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     int item = blockIdx.x;                        // chunk mode: current item
     int x = 0, hi = 0;                            // balanced mode: next granule, end of this workgroup's share
     int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
-    const int wc = blockIdx.x / units, bu = blockIdx.x % units;
+    const int wc = blockIdx.y, bu = blockIdx.x;   // balanced mode: grid = (units, shares); queue: grid = (workgroups)
     int share_q = 1, share_r = 0;                 // balanced mode: granules per share, shares with one more
     if (p.balanced) {
         const int g_first = lane < p.batch ? granules_of(lane) : 0;          // sequences 0..63
         const int incl_first = wave_scan_i32(g_first);
         int total = __builtin_amdgcn_readlane(incl_first, 63);
         for (int b0 = 64; b0 < p.batch; b0 += 64) total += wave_sum_i32(b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
-        const int shares = min((int)(gridDim.x / units), total);
+        const int shares = min((int)gridDim.y, total);
         if (p.fused && wc == 0 && tix == 0) {
             // no piece, hence no merge, ever touches a sequence without tokens: the first share writes those rows
             for (int b0 = 0; b0 < p.batch; b0 += 64) {
@@ -788,8 +789,12 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         if (p.balanced) {
             piece_end = min(before + gb, hi);
             pb = b;
-            hgb = bu / p.head_tiles;
-            ht = bu % p.head_tiles;
+            hgb = bu;
+            ht = 0;
+            if (p.head_tiles > 1) {
+                hgb = bu / p.head_tiles;
+                ht = bu % p.head_tiles;
+            }
             c_start = max(x - before - pc, 0) * kGranule;                // the first pc positions hold no tokens
             c_limit = (piece_end - before - pc) * kGranule;              // <= 0: nothing of this sequence in the share
             const int64_t slot = (int64_t)(wc + b) * units + bu;
@@ -903,7 +908,10 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // ragged batch differ in length, and a queue keeps every compute unit busy until the end.
     const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
     p.persistent = (p.counters != nullptr && !p.direct && !p.balanced && p.total_items > resident) ? 1 : 0;
-    const dim3 grid((unsigned)(p.balanced ? p.workgroups : p.persistent ? resident : p.total_items));
+    const unsigned units = (unsigned)(p.hg_blocks * p.head_tiles);
+    const dim3 grid = p.balanced ? dim3(units, (unsigned)p.workgroups / units)
+                    : p.persistent ? dim3((unsigned)resident)
+                                   : dim3(units, (unsigned)p.num_splits, (unsigned)p.batch);
     const dim3 block(64 * nw);
     // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on): two, or
     // one for the widest rows (two would not leave room for two workgroups per compute unit), in a single pass
