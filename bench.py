@@ -400,11 +400,14 @@ def main():
                 c.run()                            # first use of the stream outside the capture
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
+        # a decode step of a served model holds this call once per layer: 32 calls per graph, cycling through the pools
+        # (with two calls per graph the cost of launching the graph itself, tens of microseconds, would dominate)
+        n_in_graph = max(32, len(calls))
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):
-            for c in calls:
-                c.run()
-        reps = max(1, args.steps // len(calls))
+            for i in range(n_in_graph):
+                calls[i % len(calls)].run()
+        reps = max(3, args.steps // n_in_graph)
         for _ in range(3):
             graph.replay()
         torch.cuda.synchronize()
@@ -412,7 +415,7 @@ def main():
         for _ in range(reps):
             graph.replay()
         torch.cuda.synchronize()
-        graph_us = (time.perf_counter() - t0) * 1e6 / (reps * len(calls))
+        graph_us = (time.perf_counter() - t0) * 1e6 / (reps * n_in_graph)
 
     # ---- the un-prepared public entry point: flash_decode() validates, marshals and allocates (out, lse) per call
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, **_hints_of(args, inp))
