@@ -401,8 +401,9 @@ def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens
     to use, not as a count to force.  The reference's layer passes a fixed 32 (sp_flash_decode_layer.py:62) whatever the
     shape; results do not depend on the count, and a batch that fills the GPU on its own is not to be cut into 32 chunks
     per sequence (the Llama-3-8B shape at batch 32: 89 us as equal shares of the tokens, 135 us in 32 chunks of 128
-    tokens).  If the plan the library would choose on its own needs no more partial rows than ``kv_split`` allows it is
-    used; otherwise the count is forced.
+    tokens).  If the plan the library would choose on its own cuts the batch into equal shares (balanced mode, its answer
+    to lengths it does not know) or needs no more partial rows than ``kv_split`` allows, it is used; otherwise the count
+    is forced.
     ``flash_decode`` / ``prepare_decode`` always force."""
     if kv_split is None or kv_split <= 0:
         return -1
@@ -410,7 +411,7 @@ def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens
         return kv_split
     # the same (cached) argument block and plan that the call itself uses when the library's own plan is taken
     own = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, -1, None, None, None, "auto", None)[1]
-    return -1 if own.num_splits <= kv_split else kv_split
+    return -1 if own.balanced or own.num_splits <= kv_split else kv_split
 
 
 def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
