@@ -802,6 +802,48 @@ def test_kernel_shape_overrides_change_timing_only(cuda_device, fp8, hints):
         tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, wavefronts=3, **kw).run()
 
 
+@pytest.mark.parametrize("name,batch,n,fp8,want_balanced", [("uneven_fill", 40, 2304, False, True),
+                                                           ("fp8_chunks_one_workgroup_per_cu", 8, 4096, True, False),
+                                                           ("fp8_uneven_fill", 40, 6144, True, True)])
+def test_plans_for_alike_lengths_that_do_not_fill_the_gpu_evenly(cuda_device, name, batch, n, fp8, want_balanced):
+    """Alike lengths (the host says so): 40 x 8 units on 256 compute units would leave a quarter of them with two
+    workgroups, so the batch runs as equal shares; 8 x 4 head blocks are cut into per-sequence chunks, one workgroup
+    per compute unit, which for an fp8 cache runs eight wavefronts with one buffer each."""
+    hq, hkv, d, page = 32, 8, 128, 16
+    print(f"case alike lengths {name}", flush=True)
+    g = torch.Generator().manual_seed(batch + n)
+    lens = [n - (i % 3) for i in range(batch)]                      # within 1/32 of each other
+    pages = [(x + page - 1) // page for x in lens]
+    pool = sum(pages) + 1
+    q = torch.randn(batch, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.zeros((batch, max(pages)), dtype=torch.int32)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, x in enumerate(pages):
+        table[i, :x] = perm[at:at + x]
+        at += x
+    table, lens_t = table.to(cuda_device), _lens_t(lens, cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, torch.bfloat16), ofp8.dequant_per_head(v, vs, torch.bfloat16))
+    hints = dict(max_kv_len=max(lens), min_kv_len=min(lens))
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, **hints)
+    assert plan.balanced == want_balanced and plan.num_splits > 1, plan
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, **hints)
+    torch.cuda.synchronize()
+    rows = list(range(0, batch, max(1, batch // 8)))
+    _check(out[rows], lse[rows], q[rows], k, v, table[rows], [lens[i] for i in rows], d ** -0.5, ref_kv=ref_kv, tag=name)
+    # and against the forced single pass
+    out1, lse1 = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, kv_split=1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.float(), out1.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse, lse1, atol=1e-4, rtol=0)
+
+
 # ---- balanced mode: the kernel cuts the batch's KV ranges into equal shares from kv_lens ---------------------------
 BALANCED_CASES = {
     # name: (kv_lens, (Hq, Hkv), page, head_dim, fp8)
