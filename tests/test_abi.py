@@ -250,9 +250,9 @@ def test_plan_scales_splits_with_occupancy():
     assert p.num_splits == 1 and p.chunk_tokens >= 4096   # they fill the device: one pass, no combine
     assert p.algo == _lib.FDK_ALGO_MFMA and p.kv_heads_per_wg == 1
     # the same batch with lengths the host does not vouch for: a single pass would be as slow as its longest
-    # sequence, so the tokens are cut into equal shares (two workgroups per compute unit, two kv heads each)
+    # sequence, so the tokens are cut into equal shares (one workgroup per compute unit, two kv heads each)
     p = _plan(_args())
-    assert p.balanced == 1 and p.workgroups == 512 and p.kv_heads_per_wg == 2 and p.num_splits > 1
+    assert p.balanced == 1 and p.workgroups == 256 and p.kv_heads_per_wg == 2 and p.num_splits > 1
     assert _plan(_args(max_kv_len=4096, min_kv_len=2000)).balanced == 1
     # short contexts keep the single pass (nothing to gain from cutting them), and so do batches with four or more
     # workgroups per compute unit, which even out by themselves
@@ -279,11 +279,11 @@ def test_plan_scales_splits_with_occupancy():
     assert 6 * p_ref.num_splits <= 256 < 6 * (p_ref.num_splits + 3)
     p24 = _plan(_args(batch=24, max_pages=64, table_stride_b=64))       # 96 units, 1024 tokens
     assert p24.balanced == 0 and p24.num_splits == 2 and p24.chunk_tokens == 512
-    # few units, long context: balanced mode - two workgroups per compute unit share the KV ranges of the whole
+    # few units, long context: balanced mode - one workgroup per compute unit, they share the KV ranges of the whole
     # batch, each gets a long share, and the workspace holds (shares + batch) slots per head block
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
                          q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
-    assert p_long.balanced == 1 and p_long.workgroups == 512 and p_long.chunk_tokens >= 512
+    assert p_long.balanced == 1 and p_long.workgroups == 256 and p_long.chunk_tokens >= 512
     units = 8 // p_long.kv_heads_per_wg
     shares = p_long.workgroups // units
     rows = (shares + 4) * units * p_long.kv_heads_per_wg * 8           # group = 8 heads per tile

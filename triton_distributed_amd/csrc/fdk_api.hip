@@ -282,7 +282,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         columns < (1 << 30)) {                                            // the kernel counts granules in int32
         const int64_t gran = fdk::kBalanceGranule;
         int64_t shares = columns / (min_chunk / gran);
-        const int64_t most = 2 * (int64_t)num_cus / units_per_seq;           // two workgroups per compute unit
+        // one workgroup per compute unit: the kernel sizes such a workgroup to keep the unit's memory pipeline
+        // full by itself, and a second one only queues up behind it (measured 0.6-1.8 % slower, with twice the
+        // partial rows to merge)
+        const int64_t most = (int64_t)num_cus / units_per_seq;
         if (shares > most) shares = most;
         if (shares < 1) shares = 1;
         const int64_t share_tokens = cdiv64(columns, shares) * gran;

@@ -891,7 +891,8 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // small tiles: also per-sequence chunks that give each compute unit at most one workgroup (one-byte-per-value
     // caches cut like that measure 13-16 % faster with 8 wavefronts x 1 buffer than with 4 x 2)
     const bool shaped = single_pass || (kTileBytes <= 4096 && !p.balanced && items <= (p.num_cus > 0 ? p.num_cus : 256));
-    int nw = (p.hg_per_wg >= 4 || (shaped && kTileBytes <= 4096)) ? 8 : 4;            // wavefronts per workgroup
+    // (equal shares of the whole batch also come one workgroup to a compute unit)
+    int nw = (p.hg_per_wg >= 4 || ((shaped || p.balanced) && kTileBytes <= 4096)) ? 8 : 4;   // wavefronts per workgroup
     // a caller's override (measurements), if the kernel can run it: every kv head of the block needs a wavefront,
     // and at most four (small tiles: eight) wavefronts share a head
     if (p.tune_wavefronts >= p.hg_per_wg && p.tune_wavefronts / p.hg_per_wg <= (kTileBytes <= 4096 ? 8 : 4))
@@ -915,8 +916,9 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     const dim3 block(64 * nw);
     // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on): two, or
     // one for the widest rows (two would not leave room for two workgroups per compute unit), in a single pass
-    // whose wavefronts together hold 32 KB with one, and for long pieces with wave-uniform page numbers (two
-    // workgroups per compute unit already hold 64 KB with one: 0.6-1.4 % faster).  Short pieces, and page sizes
+    // whose wavefronts together hold 32 KB with one, and for long pieces with wave-uniform page numbers (equal
+    // shares come one workgroup to a compute unit and hold 32 KB with one buffer, chunks of a forced split come
+    // several to a unit and hold more: 0.6-1.4 % faster either way).  Short pieces, and page sizes
     // whose page numbers come by vector loads (in order with the rows), are up to 7 % faster with two.
     const bool long_pieces = pm == PM_TILE && !single_pass && p.chunk >= 512;
     const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1
