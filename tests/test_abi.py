@@ -289,13 +289,19 @@ def test_plan_scales_splits_with_occupancy():
     rows = (shares + 4) * units * p_long.kv_heads_per_wg * 8           # group = 8 heads per tile
     assert p_long.num_splits * 4 * 64 >= rows > (p_long.num_splits - 1) * 4 * 64
     assert shares * p_long.chunk_tokens >= 4 * 131072                   # the shares cover every sequence
+    # a single sequence has nothing to balance: per-sequence chunks that follow its own length
+    p_one = _plan(_args(batch=1, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
+                        q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))
+    assert p_one.balanced == 0 and p_one.chunk_floor == 64 and p_one.num_splits * (8 // p_one.kv_heads_per_wg) == 256
+    assert p_one.chunk_tokens % 16 == 0 and p_one.num_splits * p_one.chunk_tokens >= 131072
+    assert p_long.chunk_floor == 0
     # the same shape with a host-known lower bound close to the upper one: the batch is uniform, so per-sequence
     # chunks (one workgroup per compute unit) replace the balanced shares; a looser bound changes nothing
     long_kw = dict(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048, q_stride_b=64 * 128,
                    out_stride_b=64 * 128, lse_stride_b=64)
     p_uni = _plan(_args(min_kv_len=131072, **long_kw))
     assert p_uni.balanced == 0 and p_uni.num_splits * (4 * 8 // p_uni.kv_heads_per_wg) == 256
-    assert p_uni.num_splits * p_uni.chunk_tokens == 131072
+    assert p_uni.num_splits * p_uni.chunk_tokens == 131072 and p_uni.chunk_floor == 0
     assert _plan(_args(min_kv_len=131072 * 31 // 32, **long_kw)).balanced == 0
     assert _plan(_args(min_kv_len=131072 * 31 // 32 - 1, **long_kw)).balanced == 1
     assert _decode_rc(_args(min_kv_len=-1)) == _lib.FDK_ESHAPE
@@ -312,12 +318,13 @@ def test_plan_scales_splits_with_occupancy():
     # a forced split count is honoured in chunk mode: chunks are multiples of 64 tokens and cover the range
     p_forced = _plan(_args(num_splits=32))
     assert p_forced.balanced == 0 and p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
+    assert p_forced.chunk_floor == 0
     p_f4 = _plan(_args(batch=4, num_splits=5))
     assert p_f4.balanced == 0 and p_f4.chunk_tokens % 64 == 0
     assert 5 * p_f4.chunk_tokens >= 4096 > 4 * p_f4.chunk_tokens
     # the vector path splits in chunk mode
     p_v = _plan(_args(batch=4, algo=_lib.FDK_ALGO_VALU))
-    assert p_v.balanced == 0 and p_v.num_splits > 1
+    assert p_v.balanced == 0 and p_v.num_splits > 1 and p_v.chunk_floor == 0
     assert p_v.num_splits * p_v.chunk_tokens >= 4096 > (p_v.num_splits - 1) * p_v.chunk_tokens
     # fewer compute units -> no more splits / workgroups than with many
     assert _plan(_args(batch=4), cus=64).num_splits <= p4.num_splits

@@ -397,6 +397,64 @@ def test_the_lower_length_hint_selects_chunks_and_never_changes_results(cuda_dev
         tda.flash_decode(*args, max_kv_len=24000, min_kv_len=24001)
 
 
+@pytest.mark.parametrize("page", [1, 16, 64])
+def test_chunks_follow_each_sequences_own_length_when_the_host_gives_no_bounds(cuda_device, page):
+    # No length bounds at all: the plan is sized for the table's capacity and the chunks are cut on the GPU from
+    # kv_lens, as the reference cuts them (flash_decode.py:151-153).  Every row the combine merges must have been
+    # written by this call: the workspace starts out as NaN.
+    g = torch.Generator().manual_seed(97 + page)
+    hq, hkv, d, cap = 32, 8, 128, 16384
+    pages = cap // page
+    q = torch.randn(1, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pages, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pages, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.randperm(pages, generator=g).to(torch.int32).view(1, pages).to(cuda_device)
+    plan = tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5)
+    assert not plan.balanced and plan.num_splits == 64 and plan.chunk_floor == 64 and plan.chunk_tokens == 256
+    assert tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5, max_kv_len=cap,
+                                 min_kv_len=cap).chunk_floor == 0        # lengths the host vouches for: fixed chunks
+    assert tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5, kv_split=8).chunk_floor == 0
+    ws = torch.empty(plan.workspace_bytes // 4, dtype=torch.float32, device=cuda_device)
+    for n in (0, 1, 15, 16, 63, 64, 65, 1000, 64 * 64 - 1, 64 * 64, 64 * 64 + 1, 5000, 16383, cap, cap + 100):
+        print(f"page {page} kv_len {n}", flush=True)
+        ws.fill_(float("nan"))
+        lens = _lens_t([n], cuda_device)
+        out, lse = tda.flash_decode(q, k, v, table, lens, d ** -0.5, workspace=ws)
+        out1, lse1 = tda.flash_decode(q, k, v, table, lens, d ** -0.5, kv_split=1)
+        torch.cuda.synchronize()
+        if n == 0:
+            assert torch.all(out == 0) and torch.all(torch.isneginf(lse))
+            continue
+        _check(out, lse, q, k, v, table, [min(n, cap)], d ** -0.5, tag=f"own-length chunks P={page} n={n}")
+        torch.testing.assert_close(out.float(), out1.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(lse, lse1, atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("single_launch", [False, True])
+def test_own_length_chunks_of_a_short_ragged_batch_and_a_bound_that_is_too_small(cuda_device, single_launch):
+    # batches whose shares would be too short for balanced mode are cut per sequence as well; a max_kv_len below
+    # the real lengths caps the chunk, and the last split then runs to the end of its sequence
+    g = torch.Generator().manual_seed(101)
+    lens, hq, hkv, d, page = [1500, 0, 33, 700, 1], 16, 4, 128, 16
+    cap_pages = 96
+    pool = len(lens) * cap_pages
+    q = torch.randn(len(lens), hq, d, generator=g).to(torch.float16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.float16).to(cuda_device)
+    table = torch.randperm(pool, generator=g).to(torch.int32).view(len(lens), cap_pages).to(cuda_device)
+    lens_t = _lens_t(lens, cuda_device)
+    for hint in (None, 400):
+        plan = tda.get_split_kv_plan(q, k, v, table, lens_t, d ** -0.5, max_kv_len=hint)
+        assert not plan.balanced and plan.num_splits > 1 and plan.chunk_floor == 64
+        call = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=hint, single_launch=single_launch)
+        call.run()
+        torch.cuda.synchronize()
+        assert torch.all(call.out[1] == 0) and torch.all(torch.isneginf(call.lse[1]))
+        keep = [0, 2, 3, 4]
+        _check(call.out[keep], call.lse[keep], q[keep], k, v, table[keep], [lens[i] for i in keep], d ** -0.5,
+               tag=f"ragged own-length chunks hint={hint} single_launch={single_launch}")
+
+
 def test_zero_length_sequence_is_defined(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=300), cuda_device)
     lens = _lens_t([300, 0, 17], cuda_device)

@@ -11,7 +11,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
-FDK_ABI_VERSION = 7
+FDK_ABI_VERSION = 8
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -33,7 +33,7 @@ EXPORTS = (
 class FdkPlan(C.Structure):
     _fields_ = [("num_splits", C.c_int32), ("chunk_tokens", C.c_int32), ("algo", C.c_int32),
                 ("kv_heads_per_wg", C.c_int32), ("balanced", C.c_int32), ("workgroups", C.c_int32),
-                ("reserved", C.c_int32 * 2)]
+                ("chunk_floor", C.c_int32), ("reserved", C.c_int32)]
 
 
 class FdkDecodeArgs(C.Structure):

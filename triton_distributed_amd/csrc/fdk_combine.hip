@@ -55,7 +55,8 @@ __device__ __forceinline__ PartRows locate_rows(const CombineParams& p, int b, i
         // chunk mode: split c holds tokens [c*chunk, ...) - the split kernel wrote exactly the live ones
         const int kv_len = min(p.kv_lens[b], p.max_tokens);
         const int64_t row = (int64_t)b * p.hq + h;
-        r.live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);
+        const int chunk = chunk_tokens_of(kv_len, p.num_splits, p.chunk, p.chunk_floor);
+        r.live = min(p.num_splits, (kv_len + chunk - 1) / chunk);
         r.o = p.part_o + row * p.num_splits * D;
         r.lse = p.part_lse + row * p.num_splits;
         r.o_step = D;

@@ -36,6 +36,7 @@ struct SplitParams {
     int32_t batch, hq, hkv, group, head_dim;
     int32_t page_size, page_shift;  // page_shift = log2(page_size) or -1
     int32_t num_splits, chunk;
+    int32_t chunk_floor;            // chunk mode, > 0: chunks follow each sequence's own length (chunk_tokens_of)
     int32_t max_tokens;             // block_table columns * page_size: kv_len is clamped to it
     int32_t head_tiles;             // ceil(group / heads-per-workgroup)
     int32_t hg_per_wg, hg_blocks;   // kv-head groups per workgroup / workgroups along the kv-head axis
@@ -65,6 +66,7 @@ struct CombineParams {
     int64_t out_sb, out_sh, lse_sb;
     int32_t batch, hq, head_dim;
     int32_t num_splits, chunk;
+    int32_t chunk_floor;            // as in SplitParams
     int32_t max_tokens;
     int32_t out_dtype;
     int32_t pack_lse;
@@ -178,6 +180,17 @@ __device__ __forceinline__ int wave_scan_i32(int x) {
     return x;
 }
 __device__ __forceinline__ int wave_sum_i32(int x) { return __builtin_amdgcn_readlane(wave_scan_i32(x), 63); }
+
+// Chunk mode: tokens per split of a sequence that holds kv_len tokens.  chunk_floor == 0: the plan's chunk, whatever
+// the sequence holds (the plan sized it for the longest sequence the host expects).  chunk_floor > 0: the sequence's
+// own length in num_splits equal parts of whole 16-token tiles, at least chunk_floor and at most the plan's chunk
+// tokens each - as the reference cuts a sequence (flash_decode.py:151-153: cdiv(kv_len, NUM_KV_SPLITS)), so that a
+// sequence shorter than the host's bound still spreads over all the workgroups it was given.
+__device__ __forceinline__ int chunk_tokens_of(int kv_len, int num_splits, int chunk, int chunk_floor) {
+    if (chunk_floor == 0) return chunk;
+    const int even = ((kv_len + num_splits - 1) / num_splits + 15) & ~15;
+    return min(max(even, chunk_floor), chunk);
+}
 
 // Reductions over the 64 lanes with DPP only (no LDS traffic): butterflies inside each row of 16, then the row
 // results are passed down the rows (row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3), so that

@@ -318,7 +318,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         return;
     }
     const int c_end = min(c_limit, kv_len);
-    if (!p.balanced) mr.live = min(p.num_splits, (kv_len + p.chunk - 1) / p.chunk);     // chunks that hold tokens
+    if (!p.balanced && p.fused) {                                                       // chunks that hold tokens
+        const int chunk = chunk_tokens_of(kv_len, p.num_splits, p.chunk, p.chunk_floor);
+        mr.live = min(p.num_splits, (kv_len + chunk - 1) / chunk);
+    }
 
     float kscale = 1.f, vscale = 1.f;
     if (FP8) {
@@ -721,7 +724,11 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         }
         // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
         const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
-        run_piece(pb, hgb, ht, split * p.chunk, split == p.num_splits - 1 ? p.max_tokens : split * p.chunk + p.chunk,
+        // (chunks that follow the sequence's own length: the first table read then waits for kv_lens, one more
+        // round trip before the first rows - the price of not needing a length bound from the host)
+        int chunk = p.chunk;
+        if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
+        run_piece(pb, hgb, ht, split * chunk, split == p.num_splits - 1 ? p.max_tokens : split * chunk + chunk,
                   unit_row0 + (int64_t)hl * p.group * p.num_splits + split, p.num_splits,
                   MergeRows{unit_row0, 1, (int64_t)p.group * p.num_splits, p.num_splits, 0});
         return;
@@ -823,8 +830,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             wg /= p.hg_blocks;
             const int split = wg % p.num_splits;
             pb = wg / p.num_splits;
-            c_start = split * p.chunk;
-            c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + p.chunk;
+            int chunk = p.chunk;
+            if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
+            c_start = split * chunk;
+            c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + chunk;
             prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
             prow_step = p.num_splits;
             mr.live = 0;                                              // from kv_len, inside run_piece

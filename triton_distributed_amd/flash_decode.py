@@ -74,12 +74,15 @@ def _stream_handle(stream) -> int:
 class SplitKvPlan:
     """Shape-dependent launch constants (the role of the reference's ``algo_info`` dict)."""
     num_splits: int          # partial rows per (sequence, q head) the workspace holds; 1 = single pass
-    chunk_tokens: int        # tokens per split (chunk mode) / nominal tokens per workgroup (balanced mode)
+    chunk_tokens: int        # tokens per split (chunk mode; with chunk_floor: at most) / nominal tokens per
+                             # workgroup (balanced mode)
     algo: str
     workspace_bytes: int
     kv_heads_per_wg: int = 1
     balanced: bool = False   # the kernel cuts the whole batch's KV ranges into equal shares from kv_lens
     workgroups: int = 0
+    chunk_floor: int = 0     # > 0 (chunk mode): the chunks follow each sequence's own length,
+                             # clamp(ceil(kv_len / num_splits) rounded up to 16, chunk_floor, chunk_tokens) tokens
 
 
 def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -181,7 +184,7 @@ def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
     _lib.check(_LIB.fdk_plan(C.byref(a), num_cus, C.byref(plan)))
     ws = _LIB.fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits)
     return SplitKvPlan(plan.num_splits, plan.chunk_tokens, _ALGO_NAMES[plan.algo], int(ws), plan.kv_heads_per_wg,
-                       bool(plan.balanced), plan.workgroups)
+                       bool(plan.balanced), plan.workgroups, plan.chunk_floor)
 
 
 def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, soft_cap=0.0, kv_split=-1,
@@ -380,8 +383,9 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  (default ``max_pages * P``)
     min_kv_len   host-known lower bound of kv_lens (default: unknown).  A batch whose bounds lie within 1/32 of
                  each other gets whole sequences per workgroup (a single pass where they fill the GPU, else
-                 per-sequence chunks); otherwise long contexts are cut into equal shares of the tokens on the
-                 device (a single pass is as slow as its longest sequence); results never depend on it
+                 per-sequence chunks of one size); otherwise long contexts of two or more sequences are cut into
+                 equal shares of the tokens on the device (a single pass is as slow as its longest sequence) and
+                 per-sequence chunks follow each sequence's own length; results never depend on it
     k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
