@@ -44,6 +44,8 @@ def parse_args():
     ap.add_argument("--algo", default="auto", choices=["auto", "valu", "mfma"])
     ap.add_argument("--wavefronts", type=int, default=0, choices=[0, 4, 8],
                     help="measurement aid: wavefronts per workgroup of the matrix-core split kernel (0: the library's choice)")
+    ap.add_argument("--shares-per-cu", type=int, default=0, choices=[0, 1, 2, 3, 4],
+                    help="measurement aid: workgroups per compute unit of a balanced plan (0: the library's choice, 1)")
     ap.add_argument("--buffers", type=int, default=0, choices=[0, 1, 2],
                     help="measurement aid: register buffers (tiles of loads under way) per wavefront (0: the library's choice)")
     ap.add_argument("--no-hints", action="store_true",
@@ -218,7 +220,7 @@ def bench_ceiling(args):
                                                                dtype=inp.k_cache.dtype))
     pools = [(inp.k_cache, inp.v_cache), (mk(), mk())]
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
-              wavefronts=args.wavefronts, buffers=args.buffers, **_hints_of(args, inp))
+              wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
     real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
     probe = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, probe_loads=True, **kw)
              for k, v in pools]
@@ -327,6 +329,7 @@ def main():
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
                                 single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
+                                shares_per_cu=args.shares_per_cu,
                                 **_hints_of(args, inp))
              for k, v in pools]
     plan = calls[0].plan
@@ -487,6 +490,7 @@ def main():
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
             "host_length_hints": None if args.no_hints else [min(inp.kv_lens_host), max(inp.kv_lens_host)],
             "wavefronts_override": args.wavefronts or None, "buffers_override": args.buffers or None,
+            "shares_per_cu_override": args.shares_per_cu or None,
         },
         "roofline": {
             "bound": "hbm",

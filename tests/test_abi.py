@@ -40,7 +40,7 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
          offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
-         offsetof(fdk_decode_args, tune_buffers));
+         offsetof(fdk_decode_args, tune_shares_per_cu));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
@@ -57,7 +57,7 @@ int main(void) {
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
                                        ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
-                                        "tune_buffers")]
+                                        "tune_shares_per_cu")]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -221,6 +221,13 @@ def test_tuning_overrides_are_validated():
     p0, p1 = _plan(_args()), _plan(_args(tune_wavefronts=8, tune_buffers=1))
     assert (p0.num_splits, p0.balanced, p0.workgroups, p0.kv_heads_per_wg) == (p1.num_splits, p1.balanced, p1.workgroups,
                                                                                 p1.kv_heads_per_wg)
+    # workgroups per compute unit of a balanced plan: 0 (one, the library's choice) .. 4; this one is part of the plan
+    assert p0.balanced == 1 and p0.workgroups == 256
+    p2 = _plan(_args(tune_shares_per_cu=2))
+    assert p2.balanced == 1 and p2.workgroups == 512 and p2.num_splits > p0.num_splits
+    assert _plan(_args(tune_shares_per_cu=1)).workgroups == 256
+    assert _decode_rc(_args(tune_shares_per_cu=5)) == _lib.FDK_ESHAPE
+    assert _decode_rc(_args(tune_shares_per_cu=-1)) == _lib.FDK_ESHAPE
 
 
 def test_packed_output_needs_a_wider_row():

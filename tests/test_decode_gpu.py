@@ -856,6 +856,15 @@ def test_kernel_shape_overrides_change_timing_only(cuda_device, fp8, hints):
             torch.cuda.synchronize()
             torch.testing.assert_close(out.float(), out0.float(), atol=1e-2, rtol=1e-2)
             torch.testing.assert_close(lse, lse0, atol=1e-5, rtol=0)
+    for spc in (1, 2, 3):                        # workgroups per compute unit of a balanced plan
+        print(f"case overrides fp8={fp8} hints={hints} shares_per_cu={spc}", flush=True)
+        call = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, shares_per_cu=spc, **kw)
+        # (three per compute unit would be shares below 512 tokens here: the plan then drops the equal shares)
+        assert hints or call.plan.workgroups == (spc * base.plan.workgroups if spc < 3 else 0)
+        out, lse = call.run()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out.float(), out0.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(lse, lse0, atol=1e-4, rtol=0)
     with pytest.raises(Exception):
         tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, wavefronts=3, **kw).run()
 

@@ -55,6 +55,7 @@ class FdkDecodeArgs(C.Structure):
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("counters", C.c_void_p), ("counters_len", C.c_int64),
         ("tune_wavefronts", C.c_int32), ("tune_buffers", C.c_int32),
+        ("tune_shares_per_cu", C.c_int32), ("reserved_tune", C.c_int32),
     ]
 
 

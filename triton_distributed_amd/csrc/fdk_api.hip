@@ -132,6 +132,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if ((a->tune_wavefronts != 0 && a->tune_wavefronts != 4 && a->tune_wavefronts != 8) ||
         (a->tune_buffers < 0 || a->tune_buffers > 2))
         return fail(FDK_ESHAPE, "tune_wavefronts %d (0, 4, 8) / tune_buffers %d (0, 1, 2)", a->tune_wavefronts, a->tune_buffers);
+    if (a->tune_shares_per_cu < 0 || a->tune_shares_per_cu > 4)
+        return fail(FDK_ESHAPE, "tune_shares_per_cu %d (0 .. 4)", a->tune_shares_per_cu);
     if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
     if (!(a->soft_cap <= FLT_MAX)) return fail(FDK_ESHAPE, "soft_cap is not a finite number (<= 0 switches it off)");
     if (a->batch == 0) return FDK_OK;
@@ -287,7 +289,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         // one workgroup per compute unit: the kernel sizes such a workgroup to keep the unit's memory pipeline
         // full by itself, and a second one only queues up behind it (measured 0.6-1.8 % slower, with twice the
         // partial rows to merge)
-        const int64_t most = (int64_t)num_cus / units_per_seq;
+        const int64_t most = (a->tune_shares_per_cu > 0 ? a->tune_shares_per_cu : 1) * (int64_t)num_cus / units_per_seq;
         if (shares > most) shares = most;
         if (shares < 1) shares = 1;
         const int64_t share_tokens = cdiv64(columns, shares) * gran;

@@ -278,7 +278,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
-                   probe_loads=False, single_launch=False, wavefronts=0, buffers=0) -> PreparedDecode:
+                   probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -298,13 +298,17 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``static_scratch=True`` binds no workspace and no counters: the call is then to be issued with
     ``run_static()``, which keeps the split partials in the library's own static scratch.
     ``wavefronts`` (4 or 8) / ``buffers`` (1 or 2) are measurement aids: they override how the matrix-core split
-    kernel is shaped (wavefronts per workgroup, tiles of loads under way per wavefront); 0 lets the library choose."""
+    kernel is shaped (wavefronts per workgroup, tiles of loads under way per wavefront); ``shares_per_cu`` (1..4)
+    sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a, plan = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
                              k_scale, v_scale, algo, min_kv_len)
     batch, q_heads, d = q.shape
     a.tune_wavefronts, a.tune_buffers = int(wavefronts), int(buffers)
+    if shares_per_cu:
+        a.tune_shares_per_cu = int(shares_per_cu)
+        plan = _plan_of(a)                       # this one changes the plan (workgroups, workspace)
     if probe_loads:
         a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
