@@ -484,7 +484,8 @@ def main():
         "config": {
             "workload": f"{args.config}: {inp.cfg.description}",
             "algorithmic_bytes_per_call": alg_bytes,
-            "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "algo": plan.algo,
+            "num_splits": plan.num_splits, "chunk_tokens": plan.chunk_tokens, "chunk_floor": plan.chunk_floor,
+            "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "single_launch": bool(args.single_launch and plan.num_splits > 1),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
