@@ -1185,6 +1185,49 @@ def test_random_shapes_against_the_oracle(cuda_device, seed):
 
 
 @pytest.mark.parametrize("seed", list(range(24)))
+def test_random_short_sequences_in_wide_tables_against_the_oracle(cuda_device, seed):
+    # no length bounds and a table far wider than the sequences: the plan is sized for the table, the chunks follow
+    # kv_lens on the GPU (few sequences, every head size, page size and cache type)
+    rng = np.random.default_rng(7000 + seed)
+    d = int(rng.choice([64, 128, 256]))
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    group = int(rng.choice([1, 4, 8, 16]))
+    hq = hkv * group
+    page = int(rng.choice([1, 8, 16, 64]))
+    batch = int(rng.choice([1, 1, 2, 3]))
+    cap = int(rng.choice([2048, 8192, 20000]))
+    dtype = torch.bfloat16 if rng.random() < 0.5 else torch.float16
+    fp8 = bool(rng.random() < 0.3)
+    lens = [int(rng.choice([1, 17, 64, 65, 500, 1023, 1024, 1800])) for _ in range(batch)]
+    print(f"case wide table seed={seed} B={batch} {hq}q/{hkv}kv D={d} P={page} cap={cap} lens={lens} {dtype} fp8={fp8}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 2
+    q = torch.randn(batch, hq, d, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(dtype).to(cuda_device)
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    table = torch.full((batch, (cap + page - 1) // page), -1, dtype=torch.int32)     # unused columns: never followed
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    table = table.to(cuda_device)
+    ks = vs = ref_kv = None
+    if fp8:
+        k, ks = wl.quantize_kv_fp8(k)
+        v, vs = wl.quantize_kv_fp8(v)
+        ref_kv = (ofp8.dequant_per_head(k, ks, dtype), ofp8.dequant_per_head(v, vs, dtype))
+    lens_t = _lens_t(lens, cuda_device)
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, d ** -0.5)
+    assert plan.num_splits > 1 and (plan.balanced or plan.chunk_floor == 64)
+    ws = torch.full((plan.workspace_bytes // 4,), float("nan"), dtype=torch.float32, device=cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, k_scale=ks, v_scale=vs, workspace=ws)
+    torch.cuda.synchronize()
+    _check(out, lse, q, k, v, table, lens, d ** -0.5, ref_kv=ref_kv, tag=f"wide table seed {seed}")
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
 def test_random_long_and_wide_batches_against_the_oracle(cuda_device, seed):
     # the plans the small sweep above rarely reaches: balanced mode (few long sequences) and single pass with wide
     # head blocks (many short sequences)
