@@ -311,6 +311,13 @@ def test_plan_scales_splits_with_occupancy():
     assert p_uni.num_splits * p_uni.chunk_tokens == 131072 and p_uni.chunk_floor == 0
     assert _plan(_args(min_kv_len=131072 * 31 // 32, **long_kw)).balanced == 0
     assert _plan(_args(min_kv_len=131072 * 31 // 32 - 1, **long_kw)).balanced == 1
+    # alike lengths whose per-sequence chunks would leave compute units idle (22 x 4 head blocks x 2 chunks = 176
+    # workgroups on 256) get equal shares where the context is long enough to pay for them; fuller grids keep chunks
+    wide = dict(max_pages=1024, table_stride_b=1024, max_kv_len=16384, min_kv_len=16384)
+    assert _plan(_args(batch=22, **wide)).balanced == 1
+    p26 = _plan(_args(batch=26, **wide))
+    assert p26.balanced == 0 and p26.num_splits == 2 and p26.chunk_floor == 0
+    assert _plan(_args(batch=22, max_kv_len=1024, min_kv_len=1024)).balanced == 0
     assert _decode_rc(_args(min_kv_len=-1)) == _lib.FDK_ESHAPE
     assert _decode_rc(_args(max_kv_len=4096, min_kv_len=4097)) == _lib.FDK_ESHAPE
     assert _decode_rc(_args(max_kv_len=4096, min_kv_len=4096)) == 0

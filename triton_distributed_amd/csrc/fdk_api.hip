@@ -64,6 +64,7 @@ int query_cus() {
 constexpr int kChunkAlign = 64;     // granularity of the shortest chunk and of balanced shares
 constexpr int kTileAlign = 16;      // chunk boundaries fall on multiples of a 16-token tile (a tile never leaves its page)
 constexpr int kMinChunk = 64;       // shortest chunk (short contexts: latency matters more than the partials)
+constexpr double kBalancedExtraUs = 4.5;   // a balanced call against per-sequence chunks of the same batch, lengths alike
 constexpr int kMaxMinChunk = 512;   // long contexts are never split finer than this
 constexpr int kMaxSplits = 1024;
 constexpr int64_t kMaxTableTokens = (int64_t)1 << 30;
@@ -233,6 +234,8 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     //    pass runs at (fill + 1) / 2 of the even rate, fill = units / (rounds x compute units): 131 / 139 /
     //    159 us against 103 / 124 / 155 us of streaming time.
     const bool alike = a->min_kv_len > 0 && (int64_t)a->min_kv_len * 32 >= max_len * 31;
+    const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * 2.0 * a->head_dim *
+                             elem_size(a->kv_dtype) / kStreamBytesPerUs;      // what streaming the batch's cache takes
     bool rebalance = false;
     if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && units >= num_cus && batch <= kMaxBalancedBatch) {
         if (!alike) {
@@ -240,8 +243,6 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         } else if (units > num_cus) {
             const int64_t rounds = cdiv64(units, num_cus);
             const double fill = (double)units / (double)(rounds * num_cus);
-            const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * 2.0 * a->head_dim *
-                                     elem_size(a->kv_dtype) / kStreamBytesPerUs;
             rebalance = stream_us * 2.0 / (fill + 1.0) > 1.05 * (stream_us * 1.03 + kSplitOverheadUs);
         }
         if (rebalance) {
@@ -279,7 +280,18 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // needs none of that: per-sequence chunks, one workgroup per compute unit, are 2-7 % faster there.  The workspace then holds (shares + batch) slots of
     // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
     const int64_t columns = (int64_t)batch * cdiv64(max_len, fdk::kBalanceGranule);   // granules of all sequences, at most
-    const bool uniform = alike && !rebalance;
+    // Lengths that are alike, but per-sequence chunks that leave compute units idle (units x splits well below the
+    // compute units: batch 22 x 4 head blocks x 2 chunks = 176 workgroups on 256): the busy units do not make up for
+    // the idle ones - measured against equal shares of the same batch, 16384 tokens: 9 % slower at a fill of 0.69,
+    // 1 % at 0.81, level from 0.86 on - while equal shares cost about kBalancedExtraUs more per call (the pass over
+    // kv_lens before the first load, a combine that has to find its rows).
+    bool underfilled = false;
+    if (alike && may_split && !rebalance && batch > 1) {
+        const double fill = (double)(units * splits) / (double)num_cus;
+        const double slower = 0.75 * (0.82 - fill);
+        underfilled = slower > 0.0 && stream_us * slower > 1.2 * kBalancedExtraUs;
+    }
+    const bool uniform = alike && !rebalance && !underfilled;
     // (a single sequence has nothing to balance: its own length in equal chunks, below, does the same without the
     // pass over kv_lens and with a combine that knows where its rows are - 27 us against 34 us for 32768 tokens)
     if (algo == FDK_ALGO_MFMA && may_split && !uniform && batch > 1 && batch <= kMaxBalancedBatch &&
