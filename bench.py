@@ -434,7 +434,7 @@ def main():
 
     # ---- the drop-in for the reference's entry point, called the way the reference's layer calls it: no length bounds,
     # kv_split = 32 (sp_flash_decode_layer.py:62,100-110), output_combine given; fp8 caches are not part of that signature
-    ref_entry_us = None
+    ref_entry_us = ref_entry_fb_us = None
     if inp.cfg.kv_dtype != "fp8_e4m3":
         oc = torch.empty((inp.q.shape[0], inp.q.shape[1], inp.q.shape[2] + 1), dtype=inp.q.dtype, device=dev)
         ref_call = lambda i: tda.gqa_fwd_batch_decode_intra_rank(inp.q, *pools[i % len(pools)], None, None, inp.kv_lens,
@@ -447,6 +447,20 @@ def main():
             ref_call(i)
         torch.cuda.synchronize()
         ref_entry_us = (time.perf_counter() - t0) * 1e6 / n_entry
+        # the same entry point with a LengthFeedback block, as the layer mirror keeps one: each call plans with the
+        # bounds of kv_lens that the previous call's last kernel left in pinned host memory
+        fb = tda.LengthFeedback()
+        fb_call = lambda i: tda.gqa_fwd_batch_decode_intra_rank(inp.q, *pools[i % len(pools)], None, None, inp.kv_lens,
+                                                                inp.block_table, inp.sm_scale, output_combine=oc,
+                                                                kv_split=32, length_feedback=fb)
+        for i in range(5):
+            fb_call(i)
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n_entry):
+            fb_call(i)
+        torch.cuda.synchronize()
+        ref_entry_fb_us = (time.perf_counter() - t0) * 1e6 / n_entry
 
     traffic = None
     traffic_source = None
@@ -470,6 +484,7 @@ def main():
         "graph_replay_us_per_call": None if graph_us is None else round(graph_us, 2),
         "public_entry_us_per_call": round(entry_us, 2),
         "reference_entry_us_per_call": None if ref_entry_us is None else round(ref_entry_us, 2),
+        "reference_entry_with_feedback_us_per_call": None if ref_entry_fb_us is None else round(ref_entry_fb_us, 2),
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,

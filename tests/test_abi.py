@@ -40,7 +40,7 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
          offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
-         offsetof(fdk_decode_args, tune_shares_per_cu));
+         offsetof(fdk_decode_args, length_feedback));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
@@ -57,7 +57,7 @@ int main(void) {
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
                                        ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
-                                        "tune_shares_per_cu")]
+                                        "length_feedback")]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -228,6 +228,14 @@ def test_tuning_overrides_are_validated():
     assert _plan(_args(tune_shares_per_cu=1)).workgroups == 256
     assert _decode_rc(_args(tune_shares_per_cu=5)) == _lib.FDK_ESHAPE
     assert _decode_rc(_args(tune_shares_per_cu=-1)) == _lib.FDK_ESHAPE
+
+
+def test_length_feedback_pointer_is_validated():
+    assert _decode_rc(_args(length_feedback=0x20000)) == 0
+    assert _decode_rc(_args(length_feedback=0x20008)) == _lib.FDK_EALIGN
+    lib = _lib.load()
+    assert lib.fdk_length_feedback_alloc(None, None) == _lib.FDK_ENULL
+    assert lib.fdk_length_feedback_free(None) == 0
 
 
 def test_packed_output_needs_a_wider_row():

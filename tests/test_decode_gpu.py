@@ -455,6 +455,87 @@ def test_own_length_chunks_of_a_short_ragged_batch_and_a_bound_that_is_too_small
                tag=f"ragged own-length chunks hint={hint} single_launch={single_launch}")
 
 
+def test_length_feedback_reports_the_bounds_of_kv_lens_in_every_plan(cuda_device):
+    # the last kernel of a call leaves {min, max of the clamped kv_lens, call count, batch} where the host can read it
+    g = torch.Generator().manual_seed(103)
+    hq, hkv, d, page, cap_pages = 32, 8, 128, 16, 160
+    fb = tda.LengthFeedback()
+    assert fb.read() == (0, 0, 0, 0) and fb.bounds(4) == (None, None)
+    last_epoch = 0
+    for batch, lens, kw, what in [
+            (40, [2048] * 40, dict(max_kv_len=2048, min_kv_len=2048), "single pass"),
+            (4, [2500, 37, 1, 900], dict(max_kv_len=2500, min_kv_len=2400), "chunks"),
+            (4, [2500, 37, 0, 900], dict(), "equal shares"),
+            (1, [777], dict(), "own-length chunks"),
+            (3, [100, 5000, -3], dict(kv_split=7), "forced splits, lengths outside the table")]:
+        pool = batch * cap_pages
+        q = torch.randn(batch, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        table = torch.randperm(pool, generator=g).to(torch.int32).view(batch, cap_pages).to(cuda_device)
+        call = tda.prepare_decode(q, k, v, table, _lens_t(lens, cuda_device), d ** -0.5, length_feedback=fb, **kw)
+        print(f"case length feedback: {what}, plan {call.plan}", flush=True)
+        call.run()
+        torch.cuda.synchronize()
+        clamped = [min(max(n, 0), cap_pages * page) for n in lens]
+        lo, hi, epoch, nb = fb.read()
+        assert (lo, hi, nb) == (min(clamped), max(clamped), batch), what
+        assert epoch > last_epoch
+        last_epoch = epoch
+        assert fb.bounds(batch) == ((lo, hi) if lo >= 1 else (None, None)) and fb.bounds(batch + 1) == (None, None)
+        live = [i for i, n in enumerate(clamped) if n > 0]
+        _check(call.out[live], call.lse[live], q[live], k, v, table[live], [clamped[i] for i in live], d ** -0.5,
+               tag=f"length feedback {what}")
+    fb.close()
+
+
+def test_drop_in_entry_points_learn_the_length_bounds_from_the_previous_call(cuda_device):
+    # the reference's signature has no host-side lengths: with a LengthFeedback the first call runs the plan for unknown
+    # lengths, later calls the plan for the bounds the previous call left behind - same results, also after the
+    # lengths behind the tensor have changed (the bounds are then out of date for one call)
+    inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=32, kv_len=2304), cuda_device)
+    args = (inp.q, inp.k_cache, inp.v_cache, None, None, inp.kv_lens, inp.block_table, inp.sm_scale)
+    fb = tda.LengthFeedback()
+    stateless = tda.gqa_fwd_batch_decode_intra_rank(*args, kv_split=32).clone()
+    first = tda.gqa_fwd_batch_decode_intra_rank(*args, kv_split=32, length_feedback=fb).clone()
+    torch.cuda.synchronize()
+    assert torch.equal(first, stateless)                       # nothing known yet: the same plan
+    assert fb.bounds(32) == (2304, 2304)
+    plan_known = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                       max_kv_len=2304, min_kv_len=2304)
+    plan_unknown = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    assert plan_known.num_splits == 1 and plan_unknown.balanced
+    second = tda.gqa_fwd_batch_decode_intra_rank(*args, kv_split=32, length_feedback=fb).clone()
+    torch.cuda.synchronize()
+    known = torch.empty_like(second)
+    tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale, max_kv_len=2304,
+                       min_kv_len=2304, packed_out=known, want_lse=False).run()
+    torch.cuda.synchronize()
+    assert torch.equal(second, known)                          # the single pass of a caller who knows the lengths
+    torch.testing.assert_close(first[..., :-1].float(), second[..., :-1].float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(first[..., -1].float(), second[..., -1].float(), atol=3e-2, rtol=1e-2)
+    # the batch behind the tensor changes: ragged now, while the bounds still say alike
+    new_lens = [2304 - 71 * i for i in range(32)]
+    inp.kv_lens.copy_(_lens_t(new_lens, cuda_device))
+    out_ref, lse_ref = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
+    third = tda.gqa_fwd_batch_decode_intra_rank(*args, kv_split=32, length_feedback=fb).clone()
+    torch.cuda.synchronize()
+    assert fb.bounds(32) == (min(new_lens), 2304)
+    _check(out_ref, lse_ref, inp.q, inp.k_cache, inp.v_cache, inp.block_table, new_lens, inp.sm_scale, tag="ragged, no bounds")
+    torch.testing.assert_close(third[..., :-1].float(), out_ref.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(third[..., -1].float(), lse_ref, atol=3e-2, rtol=1e-2)     # lse rounded to 16 bits
+    fourth = tda.gqa_fwd_batch_decode(*args, kv_split=32, length_feedback=fb)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(fourth.float(), out_ref.float(), atol=1e-2, rtol=1e-2)
+    # the layer keeps a block of its own
+    layer = tda.SpGQAFlashDecodeAttention(0, 0, 1, 1, 32, 8, 128, 128, page_size=16, scale=inp.sm_scale, max_allowed_batch=32)
+    for _ in range(2):
+        res = layer(inp.q, inp.k_cache, inp.v_cache, inp.kv_lens[None], inp.block_table)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(res.float(), out_ref.float(), atol=1e-2, rtol=1e-2)
+    assert layer._feedback.bounds(32) == (min(new_lens), 2304)
+
+
 def test_zero_length_sequence_is_defined(cuda_device):
     inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=3, kv_len=300), cuda_device)
     lens = _lens_t([300, 0, 17], cuda_device)

@@ -8,7 +8,7 @@ imports without the library.
 import importlib
 
 __all__ = [
-    "PreparedDecode", "SplitKvPlan", "flash_decode", "flash_decode_bsnh", "get_split_kv_plan", "gqa_fwd_batch_decode",
+    "LengthFeedback", "PreparedDecode", "SplitKvPlan", "flash_decode", "flash_decode_bsnh", "get_split_kv_plan", "gqa_fwd_batch_decode",
     "gqa_fwd_batch_decode_aot", "gqa_fwd_batch_decode_intra_rank", "gqa_fwd_batch_decode_intra_rank_aot",
     "gqa_fwd_batch_decode_persistent", "gqa_fwd_batch_decode_persistent_aot",
     "inter_rank_combine", "pack_out_lse", "prepare_decode", "probe_linear_read", "qk_norm_rope_update_kvcache",

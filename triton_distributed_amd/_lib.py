@@ -26,7 +26,7 @@ FDK_STATIC_SCRATCH_BYTES = 32 << 20
 EXPORTS = (
     "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
     "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len", "fdk_kv_append",
-    "fdk_decode_static", "fdk_probe_linear_read",
+    "fdk_decode_static", "fdk_probe_linear_read", "fdk_length_feedback_alloc", "fdk_length_feedback_free",
 )
 
 
@@ -56,6 +56,7 @@ class FdkDecodeArgs(C.Structure):
         ("counters", C.c_void_p), ("counters_len", C.c_int64),
         ("tune_wavefronts", C.c_int32), ("tune_buffers", C.c_int32),
         ("tune_shares_per_cu", C.c_int32), ("reserved_tune", C.c_int32),
+        ("length_feedback", C.c_void_p),
     ]
 
 
@@ -137,6 +138,10 @@ def load() -> C.CDLL:
     lib.fdk_combine_ranks.argtypes = [C.POINTER(FdkCombineRanksArgs), C.c_void_p]
     lib.fdk_probe_linear_read.restype = C.c_int
     lib.fdk_probe_linear_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
+    lib.fdk_length_feedback_alloc.restype = C.c_int
+    lib.fdk_length_feedback_alloc.argtypes = [C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]
+    lib.fdk_length_feedback_free.restype = C.c_int
+    lib.fdk_length_feedback_free.argtypes = [C.c_void_p]
     lib.fdk_kv_append.restype = C.c_int
     lib.fdk_kv_append.argtypes = [C.POINTER(FdkKvAppendArgs), C.c_void_p]
     if lib.fdk_abi_version() != FDK_ABI_VERSION:

@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "fdk_device.h"
@@ -133,6 +134,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if ((a->tune_wavefronts != 0 && a->tune_wavefronts != 4 && a->tune_wavefronts != 8) ||
         (a->tune_buffers < 0 || a->tune_buffers > 2))
         return fail(FDK_ESHAPE, "tune_wavefronts %d (0, 4, 8) / tune_buffers %d (0, 1, 2)", a->tune_wavefronts, a->tune_buffers);
+    if (a->length_feedback && (reinterpret_cast<uintptr_t>(a->length_feedback) & 15u))
+        return fail(FDK_EALIGN, "length_feedback must be 16-byte aligned");
     if (a->tune_shares_per_cu < 0 || a->tune_shares_per_cu > 4)
         return fail(FDK_ESHAPE, "tune_shares_per_cu %d (0 .. 4)", a->tune_shares_per_cu);
     if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
@@ -413,6 +416,15 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
+    // length feedback: stored by the last kernel of the call - a single pass itself, else the combine kernel
+    static std::atomic<int32_t> epoch{0};
+    int32_t this_epoch = 0;
+    if (a->length_feedback) {
+        this_epoch = epoch.fetch_add(1) + 1;
+        if (this_epoch <= 0) { epoch.store(1); this_epoch = 1; }
+    }
+    sp.length_feedback = direct ? a->length_feedback : nullptr;
+    sp.feedback_epoch = this_epoch;
     sp.probe = (a->flags & FDK_FLAG_PROBE_LOADS) ? 1 : 0;
     if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128))
         return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path and head_dim 128");
@@ -434,6 +446,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     cp.hg_blocks = a->num_kv_heads / (sp.hg_per_wg > 0 ? sp.hg_per_wg : 1);
     cp.rows_per_slot = sp.rows_per_slot; cp.heads_per_tile = sp.heads_per_tile;
     cp.piece_cost = sp.piece_cost;
+    cp.length_feedback = a->length_feedback;
+    cp.feedback_epoch = this_epoch;
     return FDK_OK;
 }
 
@@ -614,6 +628,31 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
     p.partial_dtype = a->partial_dtype; p.out_dtype = a->out_dtype; p.packed = packed ? 1 : 0;
     int rc = fdk::launch_combine_ranks(p, reinterpret_cast<hipStream_t>(hip_stream));
     if (rc) return fail(rc, "rank combine launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return FDK_OK;
+}
+
+int fdk_length_feedback_alloc(int32_t** host, int32_t** device) {
+    if (!host || !device) return fail(FDK_ENULL, "host / device is null");
+    *host = *device = nullptr;
+    void* h = nullptr;
+    hipError_t e = hipHostMalloc(&h, 4 * sizeof(int32_t), hipHostMallocMapped);
+    if (e != hipSuccess) return fail((int)e, "hipHostMalloc: %s", hipGetErrorString(e));
+    void* d = nullptr;
+    e = hipHostGetDevicePointer(&d, h, 0);
+    if (e != hipSuccess || !d || (reinterpret_cast<uintptr_t>(d) & 15u)) {
+        (void)hipHostFree(h);
+        return fail(e != hipSuccess ? (int)e : FDK_EALIGN, "hipHostGetDevicePointer: %s", hipGetErrorString(e));
+    }
+    memset(h, 0, 4 * sizeof(int32_t));
+    *host = static_cast<int32_t*>(h);
+    *device = static_cast<int32_t*>(d);
+    return FDK_OK;
+}
+
+int fdk_length_feedback_free(int32_t* host) {
+    if (!host) return FDK_OK;
+    const hipError_t e = hipHostFree(host);
+    if (e != hipSuccess) return fail((int)e, "hipHostFree: %s", hipGetErrorString(e));
     return FDK_OK;
 }
 

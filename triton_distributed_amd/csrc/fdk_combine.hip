@@ -181,6 +181,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
         if (p.lse) p.lse[(int64_t)b * p.lse_sb + h] = lse;
         if (p.pack_lse) store_out(p.out, ob + D, lse, p.out_dtype);
     }
+    if (p.length_feedback && row == 0)
+        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
 }
 
 // Many splits: one workgroup per (sequence, head) row.  Every wavefront finds the global maximum and the sum
@@ -274,6 +276,8 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
         if (p.lse) p.lse[(int64_t)b * p.lse_sb + h] = lse;
         if (p.pack_lse) store_out(p.out, ob + D, lse, p.out_dtype);
     }
+    if (p.length_feedback && row == 0)
+        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
 }
 
 __device__ __forceinline__ float load_any(const void* base, int64_t idx, int dtype) {

@@ -48,6 +48,8 @@ struct SplitParams {
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
+    int32_t* length_feedback;       // single pass only: {min, max of the clamped kv_lens, epoch, batch} goes here
+    int32_t feedback_epoch;
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
     int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its
@@ -73,6 +75,8 @@ struct CombineParams {
     // balanced mode (see the split kernel): where the pieces of a (sequence, head) row are
     int32_t balanced, workgroups;
     int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile, piece_cost;
+    int32_t* length_feedback;       // as in SplitParams (null: nothing is stored)
+    int32_t feedback_epoch;
 };
 
 struct CombineRanksParams {
@@ -180,6 +184,26 @@ __device__ __forceinline__ int wave_scan_i32(int x) {
     return x;
 }
 __device__ __forceinline__ int wave_sum_i32(int x) { return __builtin_amdgcn_readlane(wave_scan_i32(x), 63); }
+
+// Length feedback (one wavefront): the smallest and the largest of the clamped kv_lens, for a host that cannot read
+// them otherwise.  The four values go out as one 16-byte store.
+__device__ __forceinline__ void store_length_bounds(int32_t* feedback, const int32_t* kv_lens, int batch, int max_tokens,
+                                                    int epoch, int lane) {
+    int lo = 0x7fffffff, hi = 0;
+    for (int b0 = 0; b0 < batch; b0 += 64) {
+        if (b0 + lane < batch) {
+            const int n = max(min(kv_lens[b0 + lane], max_tokens), 0);
+            lo = min(lo, n);
+            hi = max(hi, n);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        lo = min(lo, __shfl_xor(lo, off, 64));
+        hi = max(hi, __shfl_xor(hi, off, 64));
+    }
+    if (lane == 0) *reinterpret_cast<int4*>(feedback) = make_int4(lo, hi, epoch, batch);
+}
 
 // Chunk mode: tokens per split of a sequence that holds kv_len tokens.  chunk_floor == 0: the plan's chunk, whatever
 // the sequence holds (the plan sized it for the longest sequence the host expects).  chunk_floor > 0: the sequence's

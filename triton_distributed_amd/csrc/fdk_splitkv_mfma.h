@@ -731,6 +731,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         run_piece(pb, hgb, ht, split * chunk, split == p.num_splits - 1 ? p.max_tokens : split * chunk + chunk,
                   unit_row0 + (int64_t)hl * p.group * p.num_splits + split, p.num_splits,
                   MergeRows{unit_row0, 1, (int64_t)p.group * p.num_splits, p.num_splits, 0});
+        if (p.length_feedback && (blockIdx.x | blockIdx.y | blockIdx.z) == 0 && wave == 0)
+            store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
         return;
     }
     const int units = p.hg_blocks * p.head_tiles;

@@ -85,6 +85,40 @@ class SplitKvPlan:
                              # clamp(ceil(kv_len / num_splits) rounded up to 16, chunk_floor, chunk_tokens) tokens
 
 
+class LengthFeedback:
+    """Four int32 in pinned host memory that the GPU writes at the end of a decode call: the smallest and the largest
+    of the (clamped) ``kv_lens``, a call count and the batch size.  For callers whose lengths exist only on the GPU -
+    the reference's entry points take nothing else: ``bounds()`` before a later call gives ``(min_kv_len, max_kv_len)``
+    for its plan without a device synchronisation.  The bounds only size the plan: values that are out of date (the
+    batch changed since) cost time, never tokens."""
+
+    def __init__(self):
+        host, dev = C.c_void_p(), C.c_void_p()
+        _lib.check(_LIB.fdk_length_feedback_alloc(C.byref(host), C.byref(dev)))
+        self._host = host.value
+        self.device_ptr = dev.value
+        self._view = (C.c_int32 * 4).from_address(self._host)
+
+    def read(self):
+        """``(min, max, epoch, batch)`` as last written (epoch 0: never)."""
+        return tuple(self._view)
+
+    def bounds(self, batch: int):
+        """``(min_kv_len, max_kv_len)`` for a batch of this size, or ``(None, None)`` if nothing usable is there."""
+        lo, hi, epoch, nb = self._view
+        if epoch == 0 or nb != batch or lo < 1 or hi < lo:
+            return None, None
+        return lo, hi
+
+    def close(self):
+        """Free the block.  Only when no call that was given it can still be running (the GPU writes to it); a block
+        that is never closed stays allocated until the process ends (one page of pinned memory)."""
+        host, self._host = self._host, None
+        if host:
+            self._view = (C.c_int32 * 4)()
+            _lib.check(_LIB.fdk_length_feedback_free(host))
+
+
 def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
                k_scale, v_scale, algo, check_device=True, min_kv_len=None) -> FdkDecodeArgs:
     if q.dim() != 3:
@@ -278,7 +312,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    max_kv_len=None, k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
-                   probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0) -> PreparedDecode:
+                   probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0,
+                   length_feedback: Optional[LengthFeedback] = None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -299,7 +334,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``run_static()``, which keeps the split partials in the library's own static scratch.
     ``wavefronts`` (4 or 8) / ``buffers`` (1 or 2) are measurement aids: they override how the matrix-core split
     kernel is shaped (wavefronts per workgroup, tiles of loads under way per wavefront); ``shares_per_cu`` (1..4)
-    sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose."""
+    sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose.
+    ``length_feedback``: a ``LengthFeedback`` that the call's last kernel fills (see there)."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a, plan = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -309,6 +345,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     if shares_per_cu:
         a.tune_shares_per_cu = int(shares_per_cu)
         plan = _plan_of(a)                       # this one changes the plan (workgroups, workspace)
+    if length_feedback is not None:
+        a.length_feedback = length_feedback.device_ptr
     if probe_loads:
         a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
@@ -363,7 +401,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         a.counters_len = counters.numel()
     else:
         counters = None
-    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, counters)
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, counters)
     return PreparedDecode(a, plan, keep, target, lse)
 
 
@@ -404,7 +442,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     return call.run(stream)
 
 
-def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap) -> int:
+def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, lo=None, hi=None) -> int:
     """How the drop-ins for the reference's entry points read ``kv_split`` (its ``NUM_KV_SPLITS``): as the most splits
     to use, not as a count to force.  The reference's layer passes a fixed 32 (sp_flash_decode_layer.py:62) whatever the
     shape; results do not depend on the count, and a batch that fills the GPU on its own is not to be cut into 32 chunks
@@ -418,39 +456,58 @@ def _reference_kv_split(kv_split: int, q, k_cache, v_cache, block_table, kv_lens
     if not isinstance(kv_lens, torch.Tensor) or not q.is_cuda:
         return kv_split
     # the same (cached) argument block and plan that the call itself uses when the library's own plan is taken
-    own = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, -1, None, None, None, "auto", None)[1]
+    own = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, -1, hi, None, None, "auto", lo)[1]
     return -1 if own.balanced or own.num_splits <= kv_split else kv_split
+
+
+def _drop_in_bounds(q, kv_lens, fb):
+    """Length bounds for the drop-in entry points, whose signature has none: a call that is given a ``LengthFeedback``
+    leaves the smallest and the largest of ``kv_lens`` there, and the next call that is given the same block reads
+    them on the host - no synchronisation, and one call late at worst, which the plan tolerates (a decode step adds
+    one token per sequence; a batch that was recomposed runs its first call on the old bounds, slower but right)."""
+    if fb is None or not (q.is_cuda and isinstance(kv_lens, torch.Tensor) and kv_lens.dim() == 1):
+        return None, None, None
+    lo, hi = fb.bounds(kv_lens.numel())
+    return fb, lo, hi
 
 
 def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale,
                                     soft_cap=0.0, output_split=None, output_combine=None, kv_split=-1,
-                                    stream=None):
+                                    stream=None, length_feedback: Optional[LengthFeedback] = None):
     """Drop-in for the reference function of the same name (flash_decode.py:847-928).
 
     Returns ``output_combine [B, Hq, D+1]`` in q's dtype: attention output in ``[..., :D]``, lse in
-    ``[..., D]``.  ``workspace`` and ``q_lens`` are ignored as in the reference."""
+    ``[..., D]``.  ``workspace`` and ``q_lens`` are ignored as in the reference.
+    ``length_feedback`` (not in the reference): a ``LengthFeedback`` that the caller keeps for this batch; the call
+    plans with the bounds the previous call left there and leaves its own (see ``LengthFeedback``).  Without it the
+    call knows nothing about the lengths and every call plans alike."""
     batch, q_heads, d = q.shape
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
     if q.is_cuda:
         stream = _stream_handle(stream)
-    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap)
+    fb, lo, hi = _drop_in_bounds(q, kv_lens, length_feedback)
+    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, lo, hi)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), packed_out=output_combine,
-                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0,
+                          max_kv_len=hi, min_kv_len=lo, length_feedback=fb)
     call.run(stream)
     return output_combine
 
 
 def gqa_fwd_batch_decode(q, k_cache, v_cache, workspace, q_lens, kv_lens, block_table, scale, soft_cap=0.0,
-                         output_split=None, output_combine=None, kv_split=-1, stream=None):
+                         output_split=None, output_combine=None, kv_split=-1, stream=None,
+                         length_feedback: Optional[LengthFeedback] = None):
     """Drop-in for the reference function of the same name (flash_decode.py:763-844): ``[B, Hq, D]``."""
     if q.is_cuda:
         stream = _stream_handle(stream)
-    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap)
+    fb, lo, hi = _drop_in_bounds(q, kv_lens, length_feedback)
+    kv_split = _reference_kv_split(kv_split, q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap, lo, hi)
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, scale, soft_cap=soft_cap,
                           kv_split=kv_split, workspace=_as_scratch(output_split), out=output_combine,
-                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0)
+                          want_lse=False, stream_scratch=stream if q.is_cuda else None, work_queue=kv_split > 0,
+                          max_kv_len=hi, min_kv_len=lo, length_feedback=fb)
     return call.run(stream)[0]
 
 

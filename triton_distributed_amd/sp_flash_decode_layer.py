@@ -18,14 +18,14 @@ from typing import Callable, Optional
 
 import torch
 
-from .flash_decode import gqa_fwd_batch_decode_intra_rank, inter_rank_combine
+from .flash_decode import LengthFeedback, gqa_fwd_batch_decode_intra_rank, inter_rank_combine
 
 
 class SpGQAFlashDecodeAttention(torch.nn.Module):
 
     def __init__(self, rank, node, num_ranks, num_nodes, num_q_heads, num_kv_heads, q_head_dim, v_head_dim, page_size=1,
                  scale=1, soft_cap=0, max_allowed_batch=1, thrink_buffer_threshold=500, stages=20,
-                 all_gather: Optional[Callable[[torch.Tensor], torch.Tensor]] = None):
+                 all_gather: Optional[Callable[[torch.Tensor], torch.Tensor]] = None, length_feedback: bool = True):
         super().__init__()
         if q_head_dim != v_head_dim:
             raise ValueError("q_head_dim != v_head_dim is not built")
@@ -42,6 +42,12 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         self.max_allowed_batch = max_allowed_batch
         self.stages = stages
         self.all_gather = all_gather
+        # forward() gets the lengths only as a GPU tensor.  Every local decode leaves their bounds in this block and
+        # the next one plans with them (alike lengths that fill the GPU: one pass, no combine launch) - without a
+        # synchronisation and without changing results beyond the rounding of a different split; False: every call
+        # plans for unknown lengths.  Created at the first forward on a GPU.
+        self._want_feedback = bool(length_feedback)
+        self._feedback: Optional[LengthFeedback] = None
 
     def finalize(self):
         """The reference frees its symmetric buffers here (:78-80); nothing is held by this class."""
@@ -52,10 +58,13 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         assert global_kv_lens.shape[0] == self.num_ranks
         assert global_kv_lens.shape[1] == batch
         assert batch <= self.max_allowed_batch, f"Only support {self.max_allowed_batch} queries decode now"
+        if self._want_feedback and self._feedback is None and q.is_cuda:
+            with torch.cuda.device(q.device):
+                self._feedback = LengthFeedback()
         return gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch,
                                                global_kv_lens[self.rank], block_table, self.scale,
                                                soft_cap=self.soft_cap, output_combine=output_combine,
-                                               kv_split=self.kv_split)
+                                               kv_split=self.kv_split, length_feedback=self._feedback)
 
     def combine(self, all_ranks_output_combine, global_kv_lens, final_output=None):
         """Step 3: ``[R, B, Hq, D+1]`` blocks -> ``[B, Hq, D]``; ranks with ``kv_len == 0`` are skipped (:513-515)."""
