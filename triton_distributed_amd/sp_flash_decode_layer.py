@@ -58,9 +58,9 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
         assert global_kv_lens.shape[0] == self.num_ranks
         assert global_kv_lens.shape[1] == batch
         assert batch <= self.max_allowed_batch, f"Only support {self.max_allowed_batch} queries decode now"
-        if self._want_feedback and self._feedback is None and q.is_cuda:
+        if self._want_feedback and self._feedback is None and q.is_cuda and not torch.cuda.is_current_stream_capturing():
             with torch.cuda.device(q.device):
-                self._feedback = LengthFeedback()
+                self._feedback = LengthFeedback()           # (pinned host memory: not allocated under graph capture)
         return gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, self.workspace, [1] * batch,
                                                global_kv_lens[self.rank], block_table, self.scale,
                                                soft_cap=self.soft_cap, output_combine=output_combine,
