@@ -62,11 +62,17 @@ def parse_args():
                     help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
-    ap.add_argument("--op", default="decode", choices=["decode", "kv_append", "ceiling"],
+    ap.add_argument("--probe-loads", action="store_true", help="--op timeline: the load pipeline of the kernel only")
+    ap.add_argument("--rotate-heads", type=int, default=0, metavar="R",
+                    help="--op timeline: workgroup x of a sequence takes head block (x + R) mod (head blocks) - the same rows "
+                         "are then read from other XCDs")
+    ap.add_argument("--op", default="decode", choices=["decode", "kv_append", "ceiling", "timeline"],
                     help="decode: the hot path (default); kv_append: the step before it (RMSNorm + rotary + "
                          "paged append of one new token per sequence) at the same shape; ceiling: what the memory "
                          "system delivers for this configuration with no arithmetic in the way (a streaming read "
-                         "of as many bytes, and the split kernel reduced to its load pipeline) next to the kernel")
+                         "of as many bytes, and the split kernel reduced to its load pipeline) next to the kernel; "
+                         "timeline: when the wavefronts of the split kernel start, issue their first loads and finish, by "
+                         "XCD and by kv head (needs the measurement build: python -m triton_distributed_amd.build --timeline)")
     return ap.parse_args()
 
 
@@ -288,8 +294,62 @@ def _hints_of(args, inp):
     return {} if args.no_hints else dict(max_kv_len=max(inp.kv_lens_host), min_kv_len=min(inp.kv_lens_host))
 
 
+def bench_timeline(args):
+    """Per-wavefront clock readings of the matrix-core split kernel, from the library built with -DFDK_TIMELINE:
+    medians over the workgroups of each XCD and of each kv head, for ``--steps`` launches (at most 16).  With
+    ``--probe-loads`` the kernel is reduced to its load pipeline."""
+    import numpy as np
+    import torch
+    import triton_distributed_amd as tda
+    from triton_distributed_amd import workloads as wl
+
+    dev = torch.device("cuda:0")
+    inp = wl.make_inputs(_config_of(args, wl)).to(dev)
+    kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
+              wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
+    tl = torch.zeros(8 * 8 * 4096, dtype=torch.int64, device=dev)            # up to 4096 workgroups of 8 wavefronts
+    call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                              timeline=tl, probe_loads=args.probe_loads, **kw)
+    plan = call.plan
+    launches = []
+    if args.rotate_heads:
+        os.environ["FDK_TIMELINE_ROTATE_HEADS"] = str(args.rotate_heads)      # read by the measurement build at every launch
+    for rep in range(max(1, min(args.steps, 16))):
+        for _ in range(3):
+            call.run_splitkv()
+        torch.cuda.synchronize()
+        raw = tl.cpu().numpy().reshape(-1, 8)
+        raw = raw[raw[:, 0] > 0]                                             # wavefronts that wrote something
+        if raw.shape[0] == 0:
+            print("--op timeline: nothing was recorded - is FDK_LIBRARY the library built with --timeline?", file=sys.stderr)
+            sys.exit(2)
+        t0 = raw[:, 0].min()
+        us = lambda c: (raw[:, c] - t0) * 0.01                               # 100 MHz clock
+        end = np.maximum(us(2), np.where(raw[:, 3] > 0, us(3), 0.0))
+        wgs, first = np.unique(raw[:, 7], return_index=True)                 # one entry per workgroup: its last wavefront's end
+        es = np.array([end[raw[:, 7] == w].max() for w in wgs])
+        xcd, head = raw[first, 4], raw[first, 5] // max(plan.kv_heads_per_wg, 1) * max(plan.kv_heads_per_wg, 1)
+        launches.append({
+            "first_start_to_last_end_us": round(float(end.max()), 2),
+            "start_us_median": round(float(np.median(us(0))), 2),
+            "first_loads_issued_us_median": round(float(np.median(us(1)[raw[:, 1] > 0])), 2),
+            "end_us_min_median_max": [round(float(v), 2) for v in (es.min(), np.median(es), es.max())],
+            "end_us_median_by_xcd": {int(x): round(float(np.median(es[xcd == x])), 2) for x in sorted(set(xcd.tolist()))},
+            "end_us_median_by_kv_head": {int(h): round(float(np.median(es[head == h])), 2) for h in sorted(set(head.tolist()))},
+        })
+    print(json.dumps({"op": "timeline", "config": {"workload": f"{args.config}: {inp.cfg.description}",
+                                                     "num_splits": plan.num_splits, "balanced": plan.balanced,
+                                                     "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
+                                                     "load_pipeline_only": bool(args.probe_loads),
+                                                     "head_rotation": args.rotate_heads},
+                      "clock": "s_memrealtime, 100 MHz; times in us since the first wavefront's start",
+                      "launches": launches}))
+
+
 def main():
     args = parse_args()
+    if args.op == "timeline" and "FDK_LIBRARY" not in os.environ:
+        os.environ["FDK_LIBRARY"] = os.path.join(ROOT, "triton_distributed_amd", "lib", "libfdk_timeline.so")
     if args.gpus != 1:
         print(f"bench.py measures one GPU's share of the decode path; --gpus {args.gpus} is not supported "
               "(this build has no multi-GPU leg)", file=sys.stderr)
@@ -308,6 +368,8 @@ def main():
         return bench_kv_append(args)
     if args.op == "ceiling":
         return bench_ceiling(args)
+    if args.op == "timeline":
+        return bench_timeline(args)
     t_gen = time.perf_counter()
     inp_cpu = wl.make_inputs(_config_of(args, wl))
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)

@@ -40,7 +40,7 @@ int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
          offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
-         offsetof(fdk_decode_args, length_feedback));
+         offsetof(fdk_decode_args, timeline_len));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
@@ -57,7 +57,7 @@ int main(void) {
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
                                        ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
-                                        "length_feedback")]
+                                        "timeline_len")]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -233,6 +233,8 @@ def test_tuning_overrides_are_validated():
 def test_length_feedback_pointer_is_validated():
     assert _decode_rc(_args(length_feedback=0x20000)) == 0
     assert _decode_rc(_args(length_feedback=0x20008)) == _lib.FDK_EALIGN
+    assert _decode_rc(_args(timeline=0x20008, timeline_len=64)) == 0
+    assert _decode_rc(_args(timeline=0x20004, timeline_len=64)) == _lib.FDK_EALIGN
     lib = _lib.load()
     assert lib.fdk_length_feedback_alloc(None, None) == _lib.FDK_ENULL
     assert lib.fdk_length_feedback_free(None) == 0

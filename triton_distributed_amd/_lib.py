@@ -57,6 +57,7 @@ class FdkDecodeArgs(C.Structure):
         ("tune_wavefronts", C.c_int32), ("tune_buffers", C.c_int32),
         ("tune_shares_per_cu", C.c_int32), ("reserved_tune", C.c_int32),
         ("length_feedback", C.c_void_p),
+        ("timeline", C.c_void_p), ("timeline_len", C.c_int64),
     ]
 
 

@@ -136,6 +136,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         return fail(FDK_ESHAPE, "tune_wavefronts %d (0, 4, 8) / tune_buffers %d (0, 1, 2)", a->tune_wavefronts, a->tune_buffers);
     if (a->length_feedback && (reinterpret_cast<uintptr_t>(a->length_feedback) & 15u))
         return fail(FDK_EALIGN, "length_feedback must be 16-byte aligned");
+    if (a->timeline && ((reinterpret_cast<uintptr_t>(a->timeline) & 7u) || a->timeline_len < 0))
+        return fail(FDK_EALIGN, "timeline must be 8-byte aligned, timeline_len >= 0");
     if (a->tune_shares_per_cu < 0 || a->tune_shares_per_cu > 4)
         return fail(FDK_ESHAPE, "tune_shares_per_cu %d (0 .. 4)", a->tune_shares_per_cu);
     if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
@@ -425,6 +427,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     }
     sp.length_feedback = direct ? a->length_feedback : nullptr;
     sp.feedback_epoch = this_epoch;
+    sp.timeline = reinterpret_cast<long long*>(a->timeline);
+    sp.timeline_len = a->timeline ? a->timeline_len : 0;
     sp.probe = (a->flags & FDK_FLAG_PROBE_LOADS) ? 1 : 0;
     if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128))
         return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path and head_dim 128");

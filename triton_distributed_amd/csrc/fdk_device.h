@@ -50,6 +50,9 @@ struct SplitParams {
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
     int32_t* length_feedback;       // single pass only: {min, max of the clamped kv_lens, epoch, batch} goes here
     int32_t feedback_epoch;
+    long long* timeline;            // timeline build only (see the split kernel): eight int64 per wavefront
+    int64_t timeline_len;
+    int32_t timeline_rotate;        // timeline build only: rotation of the head blocks over the workgroups
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
     int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its

@@ -27,6 +27,9 @@
 #pragma once
 
 #include "fdk_device.h"
+#ifdef FDK_TIMELINE
+#include <stdlib.h>
+#endif
 
 namespace fdk {
 
@@ -38,6 +41,19 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// Timeline build (-DFDK_TIMELINE, a second library for measurements only; the product library has none of this): every
+// wavefront leaves eight int64 at p.timeline[8 * (linear workgroup * wavefronts + wavefront)] - the 100 MHz constant
+// clock at kernel entry, before the first K/V loads of its last piece, after that piece's last tile and after its
+// merge and stores (0 if the wavefront left earlier), then the XCD it ran on, the kv head, the sequence and the
+// linear workgroup index.  In that build the environment variable FDK_TIMELINE_ROTATE_HEADS=r makes workgroup x of a
+// sequence take head block (x + r) mod (head blocks) instead of x (chunk mode and single pass, one q-head tile):
+// which XCD reads which head's rows then changes, the rows themselves do not.
+#ifdef FDK_TIMELINE
+#define FDK_STAMP(i) ts[i] = (long long)__builtin_amdgcn_s_memrealtime()
+#else
+#define FDK_STAMP(i) ((void)0)
+#endif
 typedef const __attribute__((address_space(4))) int32_t* ConstI32;     // read-only for the whole kernel
 __device__ __forceinline__ ConstI32 as_const(const int32_t* p) { return (ConstI32)(uintptr_t)p; }
 
@@ -229,6 +245,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     constexpr int DB = D / 16;                 // 16-column blocks of the output
     constexpr int kScratch = 2 * kTile * RB;   // LDS bytes per wavefront: K tile + V tile; also 16 fp32 output rows
 
+#ifdef FDK_TIMELINE
+    long long ts[4] = {0, 0, 0, 0};
+#endif
+    FDK_STAMP(0);
     extern __shared__ __attribute__((aligned(16))) char lds[];      // [nw][kScratch] then m[nw][16], l[nw][16]
 
     const int lane = threadIdx.x & 63;
@@ -270,6 +290,17 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     const int kvh = hgb * nh + hl;
     const int head0 = kvh * p.group + ht * 16;
     const int heads_here = min(16, p.group - ht * 16);
+#ifdef FDK_TIMELINE
+    auto timeline_out = [&]() {
+        const int64_t w = ((int64_t)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) * nw + wave) * 8;
+        if (p.timeline && lane == 0 && w + 8 <= p.timeline_len) {
+            long long* o = p.timeline + w;
+            o[0] = ts[0]; o[1] = ts[1]; o[2] = ts[2]; o[3] = ts[3];
+            o[4] = (long long)(__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 15);        // XCC_ID
+            o[5] = kvh; o[6] = b; o[7] = (long long)(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
+        }
+    };
+#endif
 
     // Issue everything that does not depend on kv_len first, so that the dependent chain before the first K/V
     // load is as short as possible: Q^T (the B operand of S^T = K Q^T: lane (h = c, a) holds
@@ -529,6 +560,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         R rg;
         int t = tix;
         const int st = ti_n;
+        FDK_STAMP(1);
         if (t < n_full) issue_full(t, pa, rg);
         if (NBUF == 1) {
             // one register buffer: the next tile's loads go into the registers just staged
@@ -578,6 +610,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         }
     }
 
+    FDK_STAMP(2);
+#ifdef FDK_TIMELINE
+    timeline_out();
+#endif
     // ---- merge: lane groups (sum of l), then the wavefronts that share a kv head through LDS --------------
     // A wave leaves its accumulators in its own scratch as [column block][lane] float4, i.e. exactly as its lanes
     // hold them: every LDS instruction then touches one contiguous kilobyte.  The waves of a head share the
@@ -695,6 +731,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             }
         }
     }
+    FDK_STAMP(3);
+#ifdef FDK_TIMELINE
+    timeline_out();
+#endif
 
     };   // run_piece
 
@@ -718,6 +758,9 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         // (Workgroups are handed out in x-major order: neighbours still read neighbouring heads of the same tokens.)
         const int split = blockIdx.y, pb = blockIdx.z;
         int ht = 0, hgb = blockIdx.x;
+#ifdef FDK_TIMELINE
+        if (p.head_tiles == 1) hgb = (int)((blockIdx.x + (unsigned)p.timeline_rotate) % gridDim.x);
+#endif
         if (p.head_tiles > 1) {
             ht = blockIdx.x % p.head_tiles;
             hgb = blockIdx.x / p.head_tiles;
@@ -896,6 +939,12 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // workgroup and register buffers per wavefront (below) follow from the tile size; blocks of 4 or 8 kv heads
     // always take 8 wavefronts.  Measured, batch 32 x 8 kv heads x 4096 tokens: 16-bit cache 85.3 us with two
     // buffers, 81.7 us with one; fp8 cache 52.3 us with 4 wavefronts x 2 buffers, 47.1 us with 8 x 1.
+#ifdef FDK_TIMELINE
+    {
+        const char* rot = getenv("FDK_TIMELINE_ROTATE_HEADS");
+        p.timeline_rotate = rot ? atoi(rot) & 1023 : 0;
+    }
+#endif
     constexpr int kTileBytes = 2 * kTile * D * (FP8 ? 1 : 2);                    // K and V rows of one tile
     const int64_t items = (int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles;
     const bool single_pass = p.num_splits == 1 && !p.balanced;

@@ -313,7 +313,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    algo="auto", packed_out=None, want_lse=True, always_workspace=False, counters=None,
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
                    probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0,
-                   length_feedback: Optional[LengthFeedback] = None) -> PreparedDecode:
+                   length_feedback: Optional[LengthFeedback] = None, timeline: Optional[torch.Tensor] = None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -335,7 +335,9 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``wavefronts`` (4 or 8) / ``buffers`` (1 or 2) are measurement aids: they override how the matrix-core split
     kernel is shaped (wavefronts per workgroup, tiles of loads under way per wavefront); ``shares_per_cu`` (1..4)
     sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose.
-    ``length_feedback``: a ``LengthFeedback`` that the call's last kernel fills (see there)."""
+    ``length_feedback``: a ``LengthFeedback`` that the call's last kernel fills (see there).
+    ``timeline``: an int64 GPU tensor, eight values per wavefront of the split kernel; only a library built with
+    ``--timeline`` writes it (``fdk_decode_args.timeline``)."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     a, plan = _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -347,6 +349,10 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         plan = _plan_of(a)                       # this one changes the plan (workgroups, workspace)
     if length_feedback is not None:
         a.length_feedback = length_feedback.device_ptr
+    if timeline is not None:
+        if timeline.dtype != torch.int64 or not timeline.is_cuda or not timeline.is_contiguous():
+            raise ValueError("timeline must be a contiguous int64 GPU tensor")
+        a.timeline, a.timeline_len = timeline.data_ptr(), timeline.numel()
     if probe_loads:
         a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
@@ -401,7 +407,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         a.counters_len = counters.numel()
     else:
         counters = None
-    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, counters)
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, timeline, counters)
     return PreparedDecode(a, plan, keep, target, lse)
 
 
