@@ -342,7 +342,8 @@ def test_plan_scales_splits_with_occupancy():
     # a forced split count is honoured in chunk mode: chunks are multiples of 64 tokens and cover the range
     p_forced = _plan(_args(num_splits=32))
     assert p_forced.balanced == 0 and p_forced.num_splits == 32 and p_forced.chunk_tokens * 32 >= 4096
-    assert p_forced.chunk_floor == 0
+    assert p_forced.chunk_floor == 64                       # lengths unknown: the chunks follow each sequence's length
+    assert _plan(_args(num_splits=32, max_kv_len=4096, min_kv_len=4096)).chunk_floor == 0
     p_f4 = _plan(_args(batch=4, num_splits=5))
     assert p_f4.balanced == 0 and p_f4.chunk_tokens % 64 == 0
     assert 5 * p_f4.chunk_tokens >= 4096 > 4 * p_f4.chunk_tokens

@@ -413,18 +413,24 @@ def test_chunks_follow_each_sequences_own_length_when_the_host_gives_no_bounds(c
     assert not plan.balanced and plan.num_splits == 64 and plan.chunk_floor == 64 and plan.chunk_tokens == 256
     assert tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5, max_kv_len=cap,
                                  min_kv_len=cap).chunk_floor == 0        # lengths the host vouches for: fixed chunks
-    assert tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5, kv_split=8).chunk_floor == 0
+    assert tda.get_split_kv_plan(q, k, v, table, _lens_t([cap], cuda_device), d ** -0.5, kv_split=8).chunk_floor == 64
     ws = torch.empty(plan.workspace_bytes // 4, dtype=torch.float32, device=cuda_device)
+    ws32 = torch.empty_like(ws)
     for n in (0, 1, 15, 16, 63, 64, 65, 1000, 64 * 64 - 1, 64 * 64, 64 * 64 + 1, 5000, 16383, cap, cap + 100):
         print(f"page {page} kv_len {n}", flush=True)
         ws.fill_(float("nan"))
         lens = _lens_t([n], cuda_device)
         out, lse = tda.flash_decode(q, k, v, table, lens, d ** -0.5, workspace=ws)
         out1, lse1 = tda.flash_decode(q, k, v, table, lens, d ** -0.5, kv_split=1)
+        ws32.fill_(float("nan"))
+        out32, lse32 = tda.flash_decode(q, k, v, table, lens, d ** -0.5, kv_split=32, workspace=ws32)   # the reference's count
         torch.cuda.synchronize()
         if n == 0:
             assert torch.all(out == 0) and torch.all(torch.isneginf(lse))
+            assert torch.all(out32 == 0) and torch.all(torch.isneginf(lse32))
             continue
+        torch.testing.assert_close(out32.float(), out1.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(lse32, lse1, atol=1e-4, rtol=1e-5)
         _check(out, lse, q, k, v, table, [min(n, cap)], d ** -0.5, tag=f"own-length chunks P={page} n={n}")
         torch.testing.assert_close(out.float(), out1.float(), atol=1e-2, rtol=1e-2)
         torch.testing.assert_close(lse, lse1, atol=1e-4, rtol=1e-5)

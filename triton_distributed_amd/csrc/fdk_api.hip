@@ -336,9 +336,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     plan->chunk_tokens = (int32_t)chunk;
     // Lengths the host does not vouch for: the chunks follow each sequence's own length, so that a sequence far
     // below the bound (the capacity of the table, if the host gave none) still uses every workgroup it was given.
-    // The kernel then needs kv_lens before its first table read, about a microsecond: not for lengths known to
-    // be alike, and a forced split count keeps the fixed chunks that the header documents.
-    if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && splits > 1 && !alike)
+    // A forced split count is cut the same way - it is the reference's NUM_KV_SPLITS, and the reference cuts every
+    // sequence into that many parts of its own length (flash_decode.py:151-153).  Not for lengths known to be alike:
+    // the kernel then requests kv_lens and its first page numbers together.
+    if (algo == FDK_ALGO_MFMA && splits > 1 && !alike)
         plan->chunk_floor = (int32_t)(chunk < kMinChunk ? chunk : kMinChunk);
     return FDK_OK;
 }
