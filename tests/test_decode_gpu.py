@@ -1609,11 +1609,11 @@ def test_reference_entry_points_read_kv_split_as_an_upper_bound(cuda_device):
     big = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=40, kv_len=600), cuda_device)
     one = wl.make_inputs(wl.scaled_down(wl.CONFIGS["llama3_8b_b32"], batch=1, kv_len=16000), cuda_device)
     args = lambda i: (i.q, i.k_cache, i.v_cache, i.block_table, i.kv_lens, i.sm_scale, 0.0)
-    assert fd._reference_kv_split(32, *args(big)) == -1          # 40 x 8 units fill the GPU: one pass, no chunks
-    assert fd._reference_kv_split(-1, *args(big)) == -1
+    assert fd._reference_kv_split(32, *args(big))[0] == -1          # 40 x 8 units fill the GPU: one pass, no chunks
+    assert fd._reference_kv_split(-1, *args(big)) == (-1, None)
     own = tda.get_split_kv_plan(one.q, one.k_cache, one.v_cache, one.block_table, one.kv_lens)
-    assert own.num_splits > 4 and fd._reference_kv_split(4, *args(one)) == 4       # fewer than the library would take: forced
-    assert fd._reference_kv_split(1024, *args(one)) == -1
+    assert own.num_splits > 4 and fd._reference_kv_split(4, *args(one)) == (4, None)       # fewer than the library would take: forced
+    assert fd._reference_kv_split(1024, *args(one))[0] == -1
     for inp in (big, one):
         packed = tda.gqa_fwd_batch_decode_intra_rank(inp.q, inp.k_cache, inp.v_cache, None, None, inp.kv_lens,
                                                      inp.block_table, inp.sm_scale, kv_split=32)
