@@ -230,11 +230,13 @@ def test_append_then_decode_equals_attention_over_the_grown_cache(cuda_device):
     assert torch.equal(out[0].cpu().view(hkv, hq // hkv, d), qkv[0, 0, hq + hkv:][:, None].expand(hkv, hq // hkv, d))
 
 
-def test_prefill_sized_append_and_per_sequence_tables(cuda_device):
-    # many new tokens per sequence, cos / sin given per sequence ([B, S, D])
+@pytest.mark.parametrize("hq,hkv,t", [(8, 1, 300), (16, 1, 301), (20, 1, 301)])
+def test_prefill_sized_append_and_per_sequence_tables(cuda_device, hq, hkv, t):
+    # many new tokens per sequence, cos / sin given per sequence ([B, S, D]); 9000 / 15351 / 19866 head rows: grids of
+    # one, two and four rows per wavefront, the last wavefront of the larger two only partly filled
     dev = cuda_device
-    hq, hkv, d, page, t = 8, 1, 128, 16, 300
-    lens = [300, 1500, 777]
+    d, page = 128, 16
+    lens = [t, 1500, 777]
     qkv, wq, wk, table, k, v, cos, sin = _setup(31, lens, t, hq, hkv, d, page, torch.bfloat16)
     cos3 = cos[None].repeat(3, 1, 1).contiguous()
     sin3 = sin[None].repeat(3, 1, 1).contiguous()
