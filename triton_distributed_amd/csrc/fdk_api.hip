@@ -282,8 +282,9 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     // Balanced mode replaces the per-sequence chunks whenever the matrix-core path would split on its own
     // account: the kernel cuts the KV ranges of the whole batch, as kv_lens gives them, into equal shares, so
     // that a ragged batch loads every workgroup alike.  A batch the host knows to be of (nearly) uniform length
-    // needs none of that: per-sequence chunks, one workgroup per compute unit, are 2-7 % faster there.  The workspace then holds (shares + batch) slots of
-    // partial rows per (head block, head tile) unit; it is reported as rows per (sequence, q head).
+    // needs none of that: per-sequence chunks, one workgroup per compute unit, are 2-7 % faster there.  The
+    // workspace then holds (shares + batch) slots of partial rows per (head block, head tile) unit; it is reported
+    // as rows per (sequence, q head).
     const int64_t columns = (int64_t)batch * cdiv64(max_len, fdk::kBalanceGranule);   // granules of all sequences, at most
     // Lengths that are alike, but per-sequence chunks that leave compute units idle (units x splits well below the
     // compute units: batch 22 x 4 head blocks x 2 chunks = 176 workgroups on 256): the busy units do not make up for
