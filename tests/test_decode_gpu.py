@@ -675,7 +675,8 @@ def test_hip_graph_replays_follow_the_inputs(cuda_device, mode):
     lens_sets = [torch.randint(1, n_max + 1, (b,), generator=g).to(torch.int32) for _ in range(3)]
     lens_sets[1][0] = 0                                                        # an empty sequence in one replay
     lens_t = lens_sets[0].clone().to(cuda_device)
-    call = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=n_max, **kw)
+    fb = tda.LengthFeedback()           # the replays also report the bounds of the lengths they ran on
+    call = tda.prepare_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=n_max, length_feedback=fb, **kw)
     if mode == "balanced":
         assert call.plan.balanced
     elif mode == "single_pass":
@@ -698,6 +699,7 @@ def test_hip_graph_replays_follow_the_inputs(cuda_device, mode):
         want_o, want_l = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, max_kv_len=n_max, **kw)   # eager, own buffers
         torch.cuda.synchronize()
         assert torch.equal(got_o, want_o) and torch.equal(got_l, want_l), f"replay {i}"
+        assert fb.read()[:2] == (int(new_lens.min()), int(new_lens.max())) and fb.read()[3] == b, f"replay {i}"
         live = [j for j in range(b) if int(new_lens[j]) > 0]
         rows = live[:4]
         _check(got_o[rows], got_l[rows], q[rows], k, v, table[rows], [int(new_lens[j]) for j in rows], d ** -0.5,
