@@ -62,6 +62,10 @@ def parse_args():
                     help="also run a plain device copy of this many MiB three times (a kernel of known traffic, "
                          "for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget of the CPU baseline sample")
+    ap.add_argument("--kv-placement", default="staggered", choices=["staggered", "separate"],
+                    help="where the K pool and the V pool of a call lie: staggered (default) = one allocation, the V pool "
+                         "256 bytes off the K pool modulo 512, as this package's PagedKVCache allocates them "
+                         "(triton_distributed_amd.alloc_kv_pools); separate = two independent torch allocations")
     ap.add_argument("--probe-loads", action="store_true", help="--op timeline: the load pipeline of the kernel only")
     ap.add_argument("--rotate-heads", type=int, default=0, metavar="R",
                     help="--op timeline: workgroup x of a sequence takes head block (x + R) mod (head blocks) - the same rows "
@@ -203,6 +207,19 @@ def _time_launches(torch, fn, n_iter, warm=10):
     return e0.elapsed_time(e1) * 1e3 / n_iter
 
 
+def _placed(args, tda, pools):
+    """The (K, V) pools as the run wants them placed: copies into alloc_kv_pools pairs, or the tensors as they are."""
+    if args.kv_placement != "staggered":
+        return pools
+    out = []
+    for k, v in pools:
+        k2, v2 = tda.alloc_kv_pools(tuple(k.shape), k.dtype, k.device, zero=False)
+        k2.copy_(k)
+        v2.copy_(v)
+        out.append((k2, v2))
+    return out
+
+
 def bench_ceiling(args):
     """Load-only figures for one configuration, each timed like the kernel itself (events around back-to-back
     launches that cycle through two KV pools):
@@ -224,7 +241,7 @@ def bench_ceiling(args):
     mk = (lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
         torch.float8_e4m3fn)) if fp8 else (lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev,
                                                                dtype=inp.k_cache.dtype))
-    pools = [(inp.k_cache, inp.v_cache), (mk(), mk())]
+    pools = _placed(args, tda, [(inp.k_cache, inp.v_cache), (mk(), mk())])
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
               wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
     real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
@@ -308,7 +325,8 @@ def bench_timeline(args):
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
               wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
     tl = torch.zeros(8 * 8 * 4096, dtype=torch.int64, device=dev)            # up to 4096 workgroups of 8 wavefronts
-    call = tda.prepare_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+    (k_pool, v_pool), = _placed(args, tda, [(inp.k_cache, inp.v_cache)])
+    call = tda.prepare_decode(inp.q, k_pool, v_pool, inp.block_table, inp.kv_lens, inp.sm_scale,
                               timeline=tl, probe_loads=args.probe_loads, **kw)
     plan = call.plan
     launches = []
@@ -341,7 +359,7 @@ def bench_timeline(args):
                                                      "num_splits": plan.num_splits, "balanced": plan.balanced,
                                                      "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
                                                      "load_pipeline_only": bool(args.probe_loads),
-                                                     "head_rotation": args.rotate_heads},
+                                                     "head_rotation": args.rotate_heads, "kv_placement": args.kv_placement},
                       "clock": "s_memrealtime, 100 MHz; times in us since the first wavefront's start",
                       "launches": launches}))
 
@@ -388,6 +406,8 @@ def main():
         else:
             mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype)
         pools.append((mk(), mk()))
+    separate_pools = pools
+    pools = _placed(args, tda, pools)
     calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                 v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
                                 single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
@@ -435,6 +455,25 @@ def main():
     wall_s = time.perf_counter() - t0
     ms_per_step = wall_s * 1e3 / args.steps
     gbps = alg_bytes / (wall_s / args.steps) / 1e9
+
+    # ---- the same calls on independently allocated pools (the other placement), for the record -------------------
+    separate_us = None
+    if args.kv_placement == "staggered":
+        sep = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
+                                  v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
+                                  single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
+                                  shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
+               for k, v in separate_pools]
+        for i in range(min(args.warmup, 50)):
+            sep[i % len(sep)].run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            sep[i % len(sep)].run()
+        torch.cuda.synchronize()
+        separate_us = (time.perf_counter() - t0) * 1e6 / args.steps
+        del sep
+    del separate_pools
 
     # ---- dominant kernel alone (split-KV), HIP events on the launch stream ------------------------------------
     # A single-pass plan runs one kernel, the variant that writes (out, lse) itself: the events go around the call.
@@ -543,6 +582,7 @@ def main():
         "unit": "GB/s",
         "us_per_call": round(ms_per_step * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "separate_pools_us_per_call": None if separate_us is None else round(separate_us, 2),
         "graph_replay_us_per_call": None if graph_us is None else round(graph_us, 2),
         "public_entry_us_per_call": round(entry_us, 2),
         "reference_entry_us_per_call": None if ref_entry_us is None else round(ref_entry_us, 2),
@@ -565,6 +605,8 @@ def main():
             "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "single_launch": bool(args.single_launch and plan.num_splits > 1),
+            "kv_pool_placement": ("one allocation per (K, V) pair, V 256 bytes off K modulo 512 (alloc_kv_pools, as PagedKVCache "
+                                  "allocates)" if args.kv_placement == "staggered" else "two independent torch allocations"),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
             "host_length_hints": None if args.no_hints else [min(inp.kv_lens_host), max(inp.kv_lens_host)],
             "wavefronts_override": args.wavefronts or None, "buffers_override": args.buffers or None,

@@ -17,7 +17,7 @@ __all__ = [
 
 
 _LAYERS = ("SpGQAFlashDecodeAttention",)
-_HOST_ONLY = {"PagedKVCache": ".paged_kv_cache"}      # importable without the library
+_HOST_ONLY = {"PagedKVCache": ".paged_kv_cache", "alloc_kv_pools": ".paged_kv_cache"}      # importable without the library
 
 
 def _bind():
