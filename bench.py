@@ -66,6 +66,9 @@ def parse_args():
                     help="where the K pool and the V pool of a call lie: staggered (default) = one allocation, the V pool "
                          "256 bytes off the K pool modulo 512, as this package's PagedKVCache allocates them "
                          "(triton_distributed_amd.alloc_kv_pools); separate = two independent torch allocations")
+    ap.add_argument("--no-separate-leg", action="store_true",
+                    help="do not also time the calls on independently allocated pools (separate_pools_us_per_call); for "
+                         "profiler runs, whose per-kernel averages should cover one placement only")
     ap.add_argument("--probe-loads", action="store_true", help="--op timeline: the load pipeline of the kernel only")
     ap.add_argument("--rotate-heads", type=int, default=0, metavar="R",
                     help="--op timeline: workgroup x of a sequence takes head block (x + R) mod (head blocks) - the same rows "
@@ -458,7 +461,7 @@ def main():
 
     # ---- the same calls on independently allocated pools (the other placement), for the record -------------------
     separate_us = None
-    if args.kv_placement == "staggered":
+    if args.kv_placement == "staggered" and not args.no_separate_leg:
         sep = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                   v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
                                   single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
