@@ -409,14 +409,45 @@ def main():
         else:
             mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype)
         pools.append((mk(), mk()))
-    separate_pools = pools
-    pools = _placed(args, tda, pools)
-    calls = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
-                                v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
-                                single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
-                                shares_per_cu=args.shares_per_cu,
-                                **_hints_of(args, inp))
-             for k, v in pools]
+    def prepare_all(pp):
+        return [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
+                                   v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
+                                   single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
+                                   shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
+                for k, v in pp]
+
+    # ---- the calls on independently allocated pools (the other placement), for the record: timed first, then the
+    # pools move into their placed allocations one by one and the originals go back to the driver.  (Freed device
+    # memory is wiped in the background, which takes bandwidth for some milliseconds: hence before everything else,
+    # followed by a pause, and not in between the timed legs.)
+    separate_us = None
+    if args.kv_placement == "staggered":
+        if not args.no_separate_leg:
+            sep = prepare_all(pools)
+            n_warm = 0
+            t0 = time.perf_counter()
+            while n_warm < 100 or time.perf_counter() - t0 < 0.1:
+                sep[n_warm % len(sep)].run()
+                n_warm += 1
+                if n_warm % 50 == 0:
+                    torch.cuda.synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                sep[i % len(sep)].run()
+            torch.cuda.synchronize()
+            separate_us = (time.perf_counter() - t0) * 1e6 / args.steps
+            del sep
+        placed = []
+        while pools:
+            placed += _placed(args, tda, [pools.pop(0)])
+            if not placed[1:]:
+                inp.k_cache, inp.v_cache = placed[0]
+        pools = placed
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        time.sleep(0.3)
+    calls = prepare_all(pools)
     plan = calls[0].plan
     alg_bytes = inp.algorithmic_bytes()
 
@@ -458,25 +489,6 @@ def main():
     wall_s = time.perf_counter() - t0
     ms_per_step = wall_s * 1e3 / args.steps
     gbps = alg_bytes / (wall_s / args.steps) / 1e9
-
-    # ---- the same calls on independently allocated pools (the other placement), for the record -------------------
-    separate_us = None
-    if args.kv_placement == "staggered" and not args.no_separate_leg:
-        sep = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
-                                  v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
-                                  single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
-                                  shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
-               for k, v in separate_pools]
-        for i in range(min(args.warmup, 50)):
-            sep[i % len(sep)].run()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            sep[i % len(sep)].run()
-        torch.cuda.synchronize()
-        separate_us = (time.perf_counter() - t0) * 1e6 / args.steps
-        del sep
-    del separate_pools
 
     # ---- dominant kernel alone (split-KV), HIP events on the launch stream ------------------------------------
     # A single-pass plan runs one kernel, the variant that writes (out, lse) itself: the events go around the call.
