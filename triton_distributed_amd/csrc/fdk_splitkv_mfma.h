@@ -981,8 +981,12 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // several to a unit and hold more: 0.6-1.4 % faster either way).  Short pieces, and page sizes
     // whose page numbers come by vector loads (in order with the rows), are up to 7 % faster with two.
     const bool long_pieces = pm == PM_TILE && !single_pass && p.chunk >= 512;
+    // (a block of 4 or 8 kv heads of a one-byte cache is the exception: its eight wavefronts hold 32 KB with one
+    // buffer as well, but measure 1-1.5 % faster with two - batch 128 / 256 x 8 kv heads x 8192 tokens: 329.7 -> 324.7
+    // and 667.8 -> 661.5 us)
+    const bool wide_fp8 = FP8 && p.hg_per_wg >= 4;
     const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1
-                                                       : ((shaped && kTileBytes * nw >= 32768) || long_pieces));
+                                                       : ((shaped && kTileBytes * nw >= 32768 && !wide_fp8) || long_pieces));
 #define FDK_MFMA_LAUNCH(PMV, NB) \
     hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
 #define FDK_MFMA_LAUNCH_PM(NB)                                    \
