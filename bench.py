@@ -330,11 +330,9 @@ def bench_timeline(args):
     tl = torch.zeros(8 * 8 * 4096, dtype=torch.int64, device=dev)            # up to 4096 workgroups of 8 wavefronts
     (k_pool, v_pool), = _placed(args, tda, [(inp.k_cache, inp.v_cache)])
     call = tda.prepare_decode(inp.q, k_pool, v_pool, inp.block_table, inp.kv_lens, inp.sm_scale,
-                              timeline=tl, probe_loads=args.probe_loads, **kw)
+                              timeline=tl, probe_loads=args.probe_loads, rotate_heads=args.rotate_heads, **kw)
     plan = call.plan
     launches = []
-    if args.rotate_heads:
-        os.environ["FDK_TIMELINE_ROTATE_HEADS"] = str(args.rotate_heads)      # read by the measurement build at every launch
     for rep in range(max(1, min(args.steps, 16))):
         for _ in range(3):
             call.run_splitkv()

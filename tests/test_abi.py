@@ -10,13 +10,16 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "fdk.h")
+MEASURE_HEADER = os.path.join(ROOT, "include", "fdk_measure.h")
+FROZEN_HEADER = os.path.join(ROOT, "tests", "c_abi", "fdk_abi8_rev0.h")      # include/fdk.h as first released (ABI 8)
 
 from triton_distributed_amd import _lib  # noqa: E402
-from triton_distributed_amd._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkPlan  # noqa: E402
+from triton_distributed_amd._lib import (FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkMeasureArgs,  # noqa: E402
+                                         FdkPlan)
 
 
-def _declared_functions():
-    text = open(HEADER).read()
+def _declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(fdk_[a-z_]+)\s*\(", text)))
 
@@ -25,9 +28,17 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _declared_functions()
     assert set(names) == set(_lib.EXPORTS), names
-    for n in names:
+    measure = _declared_functions(MEASURE_HEADER)
+    assert set(measure) == set(_lib.MEASURE_EXPORTS), measure
+    # a caller compiled against the first release of this ABI version finds every function it was promised
+    for n in names + measure + _declared_functions(FROZEN_HEADER):
         assert hasattr(lib, n), n
     assert lib.fdk_abi_version() == _lib.FDK_ABI_VERSION
+    assert lib.fdk_abi_revision() >= _lib.FDK_ABI_REVISION
+    # the product header names no measurement aid
+    product = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for word in ("tune_", "timeline", "probe", "PROBE"):
+        assert word not in product, word
 
 
 def test_ctypes_structs_match_the_c_layout(tmp_path):
@@ -35,12 +46,13 @@ def test_ctypes_structs_match_the_c_layout(tmp_path):
     src.write_text(r'''
 #include <stdio.h>
 #include <stddef.h>
-#include "fdk.h"
+#include "fdk_measure.h"
 int main(void) {
-  printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(fdk_decode_args), offsetof(fdk_decode_args, kv_dtype),
          offsetof(fdk_decode_args, block_table), offsetof(fdk_decode_args, sm_scale),
          offsetof(fdk_decode_args, out), offsetof(fdk_decode_args, lse), offsetof(fdk_decode_args, workspace_bytes),
-         offsetof(fdk_decode_args, timeline_len));
+         offsetof(fdk_decode_args, length_feedback), offsetof(fdk_decode_args, measure),
+         sizeof(fdk_measure_args), offsetof(fdk_measure_args, rotate_heads), offsetof(fdk_measure_args, timeline_len));
   printf("%zu %zu %zu %zu\n", sizeof(fdk_combine_ranks_args), offsetof(fdk_combine_ranks_args, partial_lse),
          offsetof(fdk_combine_ranks_args, kv_lens), offsetof(fdk_combine_ranks_args, lse_stride_b_out));
   printf("%zu %zu %zu\n", sizeof(fdk_plan_t), offsetof(fdk_plan_t, balanced), offsetof(fdk_plan_t, workgroups));
@@ -57,7 +69,8 @@ int main(void) {
     got = [int(x) for x in lines[0].split()]
     want = [C.sizeof(FdkDecodeArgs)] + [getattr(FdkDecodeArgs, f).offset for f in
                                        ("kv_dtype", "block_table", "sm_scale", "out", "lse", "workspace_bytes",
-                                        "timeline_len")]
+                                        "length_feedback", "measure")] + \
+           [C.sizeof(FdkMeasureArgs), FdkMeasureArgs.rotate_heads.offset, FdkMeasureArgs.timeline_len.offset]
     assert got == want
     got = [int(x) for x in lines[1].split()]
     want = [C.sizeof(FdkCombineRanksArgs)] + [getattr(FdkCombineRanksArgs, f).offset for f in
@@ -212,29 +225,96 @@ def test_dry_run_refuses_what_a_real_call_would_refuse():
     assert _decode_rc(_args(batch=4, workspace=0x80004)) == _lib.FDK_EALIGN
 
 
+def _measured(measure_kw, **kw):
+    """An argument block that points to a measurement block (include/fdk_measure.h); the block is kept alive on it."""
+    m = FdkMeasureArgs()
+    m.struct_size = C.sizeof(FdkMeasureArgs)
+    for k, v in measure_kw.items():
+        setattr(m, k, v)
+    a = _args(**kw)
+    a.measure = C.addressof(m)
+    a._measure_block = m
+    return a
+
+
 def test_tuning_overrides_are_validated():
     # measurement aids: 0 (the library's choice), 4 or 8 wavefronts, 1 or 2 buffers; anything else is refused
     for wf, nb, rc in [(0, 0, 0), (4, 1, 0), (8, 2, 0), (8, 0, 0), (2, 0, _lib.FDK_ESHAPE), (16, 0, _lib.FDK_ESHAPE),
                        (0, 3, _lib.FDK_ESHAPE), (0, -1, _lib.FDK_ESHAPE)]:
-        assert _decode_rc(_args(tune_wavefronts=wf, tune_buffers=nb)) == rc, (wf, nb)
+        assert _decode_rc(_measured(dict(wavefronts=wf, buffers=nb))) == rc, (wf, nb)
     # they never change the plan
-    p0, p1 = _plan(_args()), _plan(_args(tune_wavefronts=8, tune_buffers=1))
+    p0, p1 = _plan(_args()), _plan(_measured(dict(wavefronts=8, buffers=1)))
     assert (p0.num_splits, p0.balanced, p0.workgroups, p0.kv_heads_per_wg) == (p1.num_splits, p1.balanced, p1.workgroups,
                                                                                 p1.kv_heads_per_wg)
     # workgroups per compute unit of a balanced plan: 0 (one, the library's choice) .. 4; this one is part of the plan
     assert p0.balanced == 1 and p0.workgroups == 256
-    p2 = _plan(_args(tune_shares_per_cu=2))
+    p2 = _plan(_measured(dict(shares_per_cu=2)))
     assert p2.balanced == 1 and p2.workgroups == 512 and p2.num_splits > p0.num_splits
-    assert _plan(_args(tune_shares_per_cu=1)).workgroups == 256
-    assert _decode_rc(_args(tune_shares_per_cu=5)) == _lib.FDK_ESHAPE
-    assert _decode_rc(_args(tune_shares_per_cu=-1)) == _lib.FDK_ESHAPE
+    assert _plan(_measured(dict(shares_per_cu=1))).workgroups == 256
+    assert _decode_rc(_measured(dict(shares_per_cu=5))) == _lib.FDK_ESHAPE
+    assert _decode_rc(_measured(dict(shares_per_cu=-1))) == _lib.FDK_ESHAPE
+    # a measurement block of another size than this library's is refused
+    bad = _measured({})
+    bad._measure_block.struct_size = 8
+    assert _decode_rc(bad) == _lib.FDK_EABI
+
+
+def test_argument_blocks_of_older_and_newer_callers():
+    """The structs only grow at the end: a caller compiled against the first release passes a smaller struct_size and
+    is served (the fields it lacks read as zero, whatever lies behind its block); what that release kept where the
+    reserved fields are now - measurement overrides - is ignored; a block larger than the library's is refused."""
+    lib = _lib.load()
+    first = FdkDecodeArgs.measure.offset                   # sizeof(fdk_decode_args) of the first release
+    a = _args(struct_size=first)
+    a.measure = 0xdeadbeef0                                # not part of the caller's block: must not be looked at
+    assert _decode_rc(a) == 0, lib.fdk_last_error()
+    assert _plan(a).num_splits == _plan(_args()).num_splits
+    old = _args(struct_size=first)
+    old.reserved0[0], old.reserved0[1], old.reserved0[2] = 16, 3, 7    # were tune_wavefronts / tune_buffers / tune_shares_per_cu
+    old.reserved1, old.reserved2 = 0x20004, -5                          # were timeline / timeline_len
+    old.flags |= 4                                                      # was the load-probe flag
+    assert _decode_rc(old) == 0, lib.fdk_last_error()
+    p_old, p_new = _plan(old), _plan(_args())
+    assert (p_old.num_splits, p_old.workgroups, p_old.balanced) == (p_new.num_splits, p_new.workgroups, p_new.balanced)
+    for size, rc in [(first - 8, _lib.FDK_EABI), (C.sizeof(FdkDecodeArgs) + 8, _lib.FDK_EABI), (0, _lib.FDK_EABI),
+                     (first + 4, 0)]:
+        assert _decode_rc(_args(struct_size=size)) == rc, size
+    assert b"struct_size" in lib.fdk_last_error() or lib.fdk_last_error() == b""
+
+
+def test_frozen_header_is_a_prefix_of_the_current_one(tmp_path):
+    """tests/c_abi/fdk_abi8_rev0.h is include/fdk.h as first released.  Every field of its structs keeps its offset
+    (or became a reserved field of the same size), its enums keep their values, and its struct sizes are the
+    smallest struct_size the library accepts."""
+    prog = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include HEADER
+#define O(f) (unsigned)offsetof(fdk_decode_args, f)
+int main(void) {
+  printf("%u %u %u %u %u %u %u %u %u %u %u\n", (unsigned)sizeof(fdk_decode_args), O(flags), O(q), O(kv_lens), O(num_splits),
+         O(sm_scale), O(out), O(workspace), O(counters_len), O(length_feedback), (unsigned)sizeof(fdk_plan_t));
+  printf("%u %u %d %d %d %d %u %u\n", (unsigned)sizeof(fdk_combine_ranks_args), (unsigned)sizeof(fdk_kv_append_args),
+         FDK_EABI, FDK_FP32, FDK_ALGO_MFMA, FDK_ABI_VERSION, FDK_FLAG_SINGLE_LAUNCH, FDK_STATIC_SCRATCH_BYTES);
+  return 0;
+}'''
+    outs = []
+    for name, header in (("old", FROZEN_HEADER), ("new", HEADER)):
+        src = tmp_path / f"{name}.c"
+        src.write_text(prog.replace("HEADER", f'"{header}"'))
+        exe = tmp_path / name
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", str(src), "-o", str(exe)], check=True)
+        outs.append([x.split() for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines()])
+    old, new = outs
+    assert old[0][1:] == new[0][1:] and old[1] == new[1]
+    assert int(old[0][0]) == FdkDecodeArgs.measure.offset and int(new[0][0]) == C.sizeof(FdkDecodeArgs)
 
 
 def test_length_feedback_pointer_is_validated():
     assert _decode_rc(_args(length_feedback=0x20000)) == 0
     assert _decode_rc(_args(length_feedback=0x20008)) == _lib.FDK_EALIGN
-    assert _decode_rc(_args(timeline=0x20008, timeline_len=64)) == 0
-    assert _decode_rc(_args(timeline=0x20004, timeline_len=64)) == _lib.FDK_EALIGN
+    assert _decode_rc(_measured(dict(timeline=0x20008, timeline_len=64))) == 0
+    assert _decode_rc(_measured(dict(timeline=0x20004, timeline_len=64))) == _lib.FDK_EALIGN
     lib = _lib.load()
     assert lib.fdk_length_feedback_alloc(None, None) == _lib.FDK_ENULL
     assert lib.fdk_length_feedback_free(None) == 0
@@ -479,10 +559,11 @@ def test_linear_read_probe_rejects_bad_arguments():
 
 def test_load_probe_flag_is_limited_to_what_is_built():
     # the load-only variant of the split kernel exists for the matrix-core path and head_dim 128
-    ok = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS)
+    ok = _measured(dict(probe_loads=1))
     assert _decode_rc(ok) == 0
-    assert _decode_rc(_args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS, algo=_lib.FDK_ALGO_VALU)) == _lib.FDK_EUNSUPPORTED
-    wide = _args(flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PROBE_LOADS, head_dim=256, q_stride_b=32 * 256, q_stride_h=256,
+    assert _decode_rc(_measured(dict(probe_loads=1), algo=_lib.FDK_ALGO_VALU)) == _lib.FDK_EUNSUPPORTED
+    assert _decode_rc(_measured(dict(probe_loads=2))) == _lib.FDK_ESHAPE
+    wide = _measured(dict(probe_loads=1), head_dim=256, q_stride_b=32 * 256, q_stride_h=256,
                  k_stride_page=16 * 8 * 256, k_stride_tok=8 * 256, k_stride_head=256, v_stride_page=16 * 8 * 256,
                  v_stride_tok=8 * 256, v_stride_head=256, out_stride_b=32 * 256, out_stride_h=256)
     assert _decode_rc(wide) == _lib.FDK_EUNSUPPORTED

@@ -1,4 +1,4 @@
-"""ctypes binding of libfdk.so (declarations: include/fdk.h).
+"""ctypes binding of libfdk.so (declarations: include/fdk.h, measurement aids: include/fdk_measure.h).
 
 The library is loaded from ``triton_distributed_amd/lib/libfdk.so``.  There is no fallback: if the file
 is missing or a symbol is absent, importing the decode entry points raises.
@@ -12,6 +12,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
 FDK_ABI_VERSION = 8
+FDK_ABI_REVISION = 1      # the library may be newer (its structs only grow at the end), never older
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -20,14 +21,17 @@ FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK
 # fdk_algo
 FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
 # flags
-FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_PROBE_LOADS, FDK_FLAG_SINGLE_LAUNCH = 1, 2, 4, 8
+FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_SINGLE_LAUNCH = 1, 2, 8
 FDK_STATIC_SCRATCH_BYTES = 32 << 20
 
+# declared in include/fdk.h
 EXPORTS = (
-    "fdk_abi_version", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
+    "fdk_abi_version", "fdk_abi_revision", "fdk_last_error", "fdk_device_cus", "fdk_plan", "fdk_workspace_bytes",
     "fdk_decode", "fdk_decode_splitkv", "fdk_combine", "fdk_combine_ranks", "fdk_counters_len", "fdk_kv_append",
-    "fdk_decode_static", "fdk_probe_linear_read", "fdk_length_feedback_alloc", "fdk_length_feedback_free",
+    "fdk_decode_static", "fdk_length_feedback_alloc", "fdk_length_feedback_free",
 )
+# declared in include/fdk_measure.h
+MEASURE_EXPORTS = ("fdk_probe_linear_read",)
 
 
 class FdkPlan(C.Structure):
@@ -54,9 +58,18 @@ class FdkDecodeArgs(C.Structure):
         ("lse", C.c_void_p), ("lse_stride_b", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("counters", C.c_void_p), ("counters_len", C.c_int64),
-        ("tune_wavefronts", C.c_int32), ("tune_buffers", C.c_int32),
-        ("tune_shares_per_cu", C.c_int32), ("reserved_tune", C.c_int32),
+        ("reserved0", C.c_int32 * 4),
         ("length_feedback", C.c_void_p),
+        ("reserved1", C.c_void_p), ("reserved2", C.c_int64),
+        ("measure", C.c_void_p),           # FdkMeasureArgs*, null in product use
+    ]
+
+
+class FdkMeasureArgs(C.Structure):
+    """include/fdk_measure.h: overrides and probes of the benchmark; never changes a result."""
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("probe_loads", C.c_uint32),
+        ("wavefronts", C.c_int32), ("buffers", C.c_int32), ("shares_per_cu", C.c_int32), ("rotate_heads", C.c_int32),
         ("timeline", C.c_void_p), ("timeline_len", C.c_int64),
     ]
 
@@ -116,11 +129,13 @@ def load() -> C.CDLL:
             f"{path} not found: build it with `python -m triton_distributed_amd.build` (hipcc, gfx950). "
             "There is no fallback implementation.")
     lib = C.CDLL(path)
-    for name in EXPORTS:
+    for name in EXPORTS + MEASURE_EXPORTS:
         if not hasattr(lib, name):
             raise ImportError(f"{path} does not export {name}")
     lib.fdk_abi_version.restype = C.c_int
     lib.fdk_abi_version.argtypes = []
+    lib.fdk_abi_revision.restype = C.c_int
+    lib.fdk_abi_revision.argtypes = []
     lib.fdk_last_error.restype = C.c_char_p
     lib.fdk_last_error.argtypes = []
     lib.fdk_device_cus.restype = C.c_int
@@ -145,8 +160,9 @@ def load() -> C.CDLL:
     lib.fdk_length_feedback_free.argtypes = [C.c_void_p]
     lib.fdk_kv_append.restype = C.c_int
     lib.fdk_kv_append.argtypes = [C.POINTER(FdkKvAppendArgs), C.c_void_p]
-    if lib.fdk_abi_version() != FDK_ABI_VERSION:
-        raise ImportError(f"{path}: ABI version {lib.fdk_abi_version()} != {FDK_ABI_VERSION}")
+    if lib.fdk_abi_version() != FDK_ABI_VERSION or lib.fdk_abi_revision() < FDK_ABI_REVISION:
+        raise ImportError(f"{path}: ABI {lib.fdk_abi_version()}.{lib.fdk_abi_revision()}, this package needs "
+                          f"{FDK_ABI_VERSION}.{FDK_ABI_REVISION} or a later revision")
     _lib = lib
     return lib
 

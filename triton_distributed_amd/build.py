@@ -6,8 +6,8 @@ Python host only ever loads the finished file.
 
 ``--timeline`` builds ``lib/libfdk_timeline.so`` instead: the same sources with ``-DFDK_TIMELINE``, whose
 matrix-core split kernel records when every wavefront started, issued its first loads and finished
-(``fdk_decode_args.timeline``).  A measurement aid (``bench.py --op timeline`` loads it through the
-``FDK_LIBRARY`` environment variable); nothing else uses it.
+(``fdk_measure_args.timeline``, include/fdk_measure.h).  A measurement aid (``bench.py --op timeline`` loads it
+through the ``FDK_LIBRARY`` environment variable); nothing else uses it, and ``--all`` builds both.
 """
 from __future__ import annotations
 

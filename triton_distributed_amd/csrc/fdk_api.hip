@@ -9,6 +9,7 @@
 #include <atomic>
 #include <mutex>
 
+#include "../../include/fdk_measure.h"
 #include "fdk_device.h"
 
 namespace {
@@ -79,7 +80,8 @@ constexpr double kSplitOverheadUs = 7.0;      // partial rows + combine launch o
 
 // Scratch of fdk_decode_static: one copy per GPU, part of the loaded code object, never allocated or freed.
 constexpr size_t kStaticScratchBytes = FDK_STATIC_SCRATCH_BYTES;
-static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+// (256 more bytes behind it: where the streaming-read probe's checksum would go)
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes + 256];
 
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
@@ -104,10 +106,45 @@ int static_scratch_of_current_device(void** ptr) {
     return FDK_OK;
 }
 
+// The argument structs only grow at the end.  A caller's block is copied into one of this library's layout: the
+// fields it does not have read as zero.  Blocks smaller than the first revision's or larger than this library's
+// are refused.
+template <typename T>
+int adopt(const void* src, uint32_t struct_size, size_t first_revision_size, const char* what, T* dst) {
+    if (struct_size < first_revision_size || struct_size > sizeof(T))
+        return fail(FDK_EABI, "%s.struct_size %u outside [%zu, %zu]: built against another ABI line", what, struct_size,
+                    first_revision_size, sizeof(T));
+    memset(static_cast<void*>(dst), 0, sizeof(T));
+    memcpy(static_cast<void*>(dst), src, struct_size);
+    dst->struct_size = (uint32_t)sizeof(T);
+    return FDK_OK;
+}
+
+// A decode call's arguments in this library's layout, with the measurement block (all zero unless the caller
+// passed one) beside them; a.measure points at m or is null.
+struct Call {
+    fdk_decode_args a;
+    fdk_measure_args m;
+};
+
+constexpr size_t kDecodeArgsFirstRevision = offsetof(fdk_decode_args, measure);
+constexpr size_t kMeasureArgsFirstRevision = sizeof(fdk_measure_args);
+
+int adopt_call(const fdk_decode_args* args, Call* c) {
+    if (!args) return fail(FDK_ENULL, "args is null");
+    int rc = adopt(args, args->struct_size, kDecodeArgsFirstRevision, "fdk_decode_args", &c->a);
+    if (rc) return rc;
+    memset(&c->m, 0, sizeof(c->m));
+    if (c->a.measure) {
+        rc = adopt(c->a.measure, c->a.measure->struct_size, kMeasureArgsFirstRevision, "fdk_measure_args", &c->m);
+        if (rc) return rc;
+        c->a.measure = &c->m;
+    }
+    return FDK_OK;
+}
+
+// (a: a block in this library's layout, from adopt_call)
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
-    if (!a) return fail(FDK_ENULL, "args is null");
-    if (a->struct_size != sizeof(fdk_decode_args))
-        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_decode_args));
     if (a->batch < 0) return fail(FDK_ESHAPE, "batch %d < 0", a->batch);
     if (a->num_q_heads <= 0 || a->num_kv_heads <= 0)
         return fail(FDK_ESHAPE, "head counts must be positive (Hq=%d, Hkv=%d)", a->num_q_heads, a->num_kv_heads);
@@ -131,15 +168,17 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if (a->kv_dtype != a->q_dtype && a->kv_dtype != FDK_FP8_E4M3)
         return fail(FDK_EUNSUPPORTED, "kv_dtype %d must equal q_dtype or be fp8_e4m3", a->kv_dtype);
     if (a->algo < FDK_ALGO_AUTO || a->algo > FDK_ALGO_MFMA) return fail(FDK_EUNSUPPORTED, "algo %d", a->algo);
-    if ((a->tune_wavefronts != 0 && a->tune_wavefronts != 4 && a->tune_wavefronts != 8) ||
-        (a->tune_buffers < 0 || a->tune_buffers > 2))
-        return fail(FDK_ESHAPE, "tune_wavefronts %d (0, 4, 8) / tune_buffers %d (0, 1, 2)", a->tune_wavefronts, a->tune_buffers);
     if (a->length_feedback && (reinterpret_cast<uintptr_t>(a->length_feedback) & 15u))
         return fail(FDK_EALIGN, "length_feedback must be 16-byte aligned");
-    if (a->timeline && ((reinterpret_cast<uintptr_t>(a->timeline) & 7u) || a->timeline_len < 0))
-        return fail(FDK_EALIGN, "timeline must be 8-byte aligned, timeline_len >= 0");
-    if (a->tune_shares_per_cu < 0 || a->tune_shares_per_cu > 4)
-        return fail(FDK_ESHAPE, "tune_shares_per_cu %d (0 .. 4)", a->tune_shares_per_cu);
+    if (const fdk_measure_args* m = a->measure) {
+        if ((m->wavefronts != 0 && m->wavefronts != 4 && m->wavefronts != 8) || m->buffers < 0 || m->buffers > 2)
+            return fail(FDK_ESHAPE, "measure: wavefronts %d (0, 4, 8) / buffers %d (0, 1, 2)", m->wavefronts, m->buffers);
+        if (m->shares_per_cu < 0 || m->shares_per_cu > 4)
+            return fail(FDK_ESHAPE, "measure: shares_per_cu %d (0 .. 4)", m->shares_per_cu);
+        if (m->probe_loads > 1) return fail(FDK_ESHAPE, "measure: probe_loads %u (0, 1)", m->probe_loads);
+        if (m->timeline && ((reinterpret_cast<uintptr_t>(m->timeline) & 7u) || m->timeline_len < 0))
+            return fail(FDK_EALIGN, "measure: timeline must be 8-byte aligned, timeline_len >= 0");
+    }
     if (!(fabsf(a->sm_scale) <= FLT_MAX)) return fail(FDK_ESHAPE, "sm_scale is not finite");
     if (!(a->soft_cap <= FLT_MAX)) return fail(FDK_ESHAPE, "soft_cap is not a finite number (<= 0 switches it off)");
     if (a->batch == 0) return FDK_OK;
@@ -307,7 +346,8 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         // one workgroup per compute unit: the kernel sizes such a workgroup to keep the unit's memory pipeline
         // full by itself, and a second one only queues up behind it (measured 0.6-1.8 % slower, with twice the
         // partial rows to merge)
-        const int64_t most = (a->tune_shares_per_cu > 0 ? a->tune_shares_per_cu : 1) * (int64_t)num_cus / units_per_seq;
+        const int shares_per_cu = a->measure && a->measure->shares_per_cu > 0 ? a->measure->shares_per_cu : 1;
+        const int64_t most = shares_per_cu * (int64_t)num_cus / units_per_seq;
         if (shares > most) shares = most;
         if (shares < 1) shares = 1;
         const int64_t share_tokens = cdiv64(columns, shares) * gran;
@@ -415,12 +455,14 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.heads_per_tile = sp.group < 16 ? sp.group : 16;
     sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
     sp.piece_cost = sp.balanced ? piece_cost_granules(a, sp.hg_per_wg) : 0;
-    sp.tune_wavefronts = a->tune_wavefronts;
-    sp.tune_buffers = a->tune_buffers;
+    const fdk_measure_args* const ms = a->measure;
+    sp.tune_wavefronts = ms ? ms->wavefronts : 0;
+    sp.tune_buffers = ms ? ms->buffers : 0;
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
-    // length feedback: stored by the last kernel of the call - a single pass itself, else the combine kernel
+    // length feedback: stored by the last kernel of the call - a single pass (or the single-launch form) itself,
+    // else the combine kernel
     static std::atomic<int32_t> epoch{0};
     int32_t this_epoch = 0;
     if (a->length_feedback) {
@@ -429,11 +471,12 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     }
     sp.length_feedback = direct ? a->length_feedback : nullptr;
     sp.feedback_epoch = this_epoch;
-    sp.timeline = reinterpret_cast<long long*>(a->timeline);
-    sp.timeline_len = a->timeline ? a->timeline_len : 0;
-    sp.probe = (a->flags & FDK_FLAG_PROBE_LOADS) ? 1 : 0;
+    sp.timeline = ms ? reinterpret_cast<long long*>(ms->timeline) : nullptr;
+    sp.timeline_len = ms && ms->timeline ? ms->timeline_len : 0;
+    sp.timeline_rotate = ms ? ms->rotate_heads & 1023 : 0;
+    sp.probe = ms && ms->probe_loads ? 1 : 0;
     if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128))
-        return fail(FDK_EUNSUPPORTED, "FDK_FLAG_PROBE_LOADS: built for the matrix-core path and head_dim 128");
+        return fail(FDK_EUNSUPPORTED, "measure: probe_loads is built for the matrix-core path and head_dim 128");
     sp.scale_log2 = a->sm_scale * fdk::kLog2e;
     sp.soft_cap = a->soft_cap > 0.f ? a->soft_cap : 0.f;
     sp.sm_scale = a->sm_scale;
@@ -490,6 +533,7 @@ int decode_impl(const fdk_decode_args* args, void* hip_stream) {
         if ((args->flags & FDK_FLAG_SINGLE_LAUNCH) && ws_need < ((size_t)1 << 32)) {
             r.sp.fused = 1;
             r.sp.ws_bytes = (uint32_t)ws_need;
+            r.sp.length_feedback = args->length_feedback;        // no combine follows: the split kernel stores it
         }
     }
     if (dry) return FDK_OK;
@@ -508,12 +552,15 @@ extern "C" {
 
 int fdk_abi_version(void) { return FDK_ABI_VERSION; }
 
+int fdk_abi_revision(void) { return FDK_ABI_REVISION; }
+
 const char* fdk_last_error(void) { return g_err; }
 
 int fdk_device_cus(void) { return query_cus(); }
 
 int64_t fdk_counters_len(const fdk_decode_args* a) {
-    if (!a || a->batch <= 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads) return 0;
+    // (reads fields of the first revision only: no need to adopt the block)
+    if (!a || a->struct_size < kDecodeArgsFirstRevision || a->batch <= 0 || a->num_q_heads <= 0 || a->num_kv_heads <= 0 || a->num_q_heads % a->num_kv_heads) return 0;
     // queue head, finished-workgroup count, then one ticket per (sequence, kv head, tile of 16 q heads): an upper
     // bound of the (sequence, head block, head tile) units of any plan
     const int64_t group = a->num_q_heads / a->num_kv_heads;
@@ -529,23 +576,34 @@ size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim,
     return (size_t)bytes & ~(size_t)255;
 }
 
-int fdk_plan(const fdk_decode_args* args, int num_cus, fdk_plan_t* plan) {
+int fdk_plan(const fdk_decode_args* caller_args, int num_cus, fdk_plan_t* plan) {
     g_err[0] = 0;
     if (!plan) return fail(FDK_ENULL, "plan is null");
-    int rc = validate(args, false, false);
+    Call call;
+    int rc = adopt_call(caller_args, &call);
+    if (rc) return rc;
+    const fdk_decode_args* args = &call.a;
+    rc = validate(args, false, false);
     if (rc) return rc;
     if (num_cus <= 0 && (args->flags & FDK_FLAG_DRY_RUN)) num_cus = kDryRunCus;
     return make_plan(args, num_cus, plan);
 }
 
-int fdk_decode(const fdk_decode_args* args, void* hip_stream) {
+int fdk_decode(const fdk_decode_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    return decode_impl(args, hip_stream);
+    Call call;
+    const int rc = adopt_call(caller_args, &call);
+    if (rc) return rc;
+    return decode_impl(&call.a, hip_stream);
 }
 
-int fdk_decode_static(const fdk_decode_args* args, void* hip_stream) {
+int fdk_decode_static(const fdk_decode_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    int rc = validate(args, true, false);
+    Call call;
+    int rc = adopt_call(caller_args, &call);
+    if (rc) return rc;
+    const fdk_decode_args* args = &call.a;
+    rc = validate(args, true, false);
     if (rc) return rc;
     if (args->batch == 0) return FDK_OK;
     const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
@@ -574,9 +632,13 @@ int fdk_decode_static(const fdk_decode_args* args, void* hip_stream) {
     return decode_impl(&a, hip_stream);
 }
 
-int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {
+int fdk_decode_splitkv(const fdk_decode_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    int rc = validate(args, false, true);
+    Call call;
+    int rc = adopt_call(caller_args, &call);
+    if (rc) return rc;
+    const fdk_decode_args* args = &call.a;
+    rc = validate(args, false, true);
     if (rc) return rc;
     if (args->batch == 0) return FDK_OK;
     const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
@@ -586,9 +648,13 @@ int fdk_decode_splitkv(const fdk_decode_args* args, void* hip_stream) {
     return launch_split(args, r, reinterpret_cast<hipStream_t>(hip_stream));
 }
 
-int fdk_combine(const fdk_decode_args* args, void* hip_stream) {
+int fdk_combine(const fdk_decode_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    int rc = validate(args, true, true);
+    Call call;
+    int rc = adopt_call(caller_args, &call);
+    if (rc) return rc;
+    const fdk_decode_args* args = &call.a;
+    rc = validate(args, true, true);
     if (rc) return rc;
     if (args->batch == 0) return FDK_OK;
     const bool dry = (args->flags & FDK_FLAG_DRY_RUN) != 0;
@@ -600,11 +666,13 @@ int fdk_combine(const fdk_decode_args* args, void* hip_stream) {
     return FDK_OK;
 }
 
-int fdk_combine_ranks(const fdk_combine_ranks_args* a, void* hip_stream) {
+int fdk_combine_ranks(const fdk_combine_ranks_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    if (!a) return fail(FDK_ENULL, "args is null");
-    if (a->struct_size != sizeof(fdk_combine_ranks_args))
-        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_combine_ranks_args));
+    if (!caller_args) return fail(FDK_ENULL, "args is null");
+    fdk_combine_ranks_args local;
+    if (int rc = adopt(caller_args, caller_args->struct_size, sizeof(fdk_combine_ranks_args), "fdk_combine_ranks_args", &local))
+        return rc;
+    const fdk_combine_ranks_args* a = &local;
     if (a->num_ranks <= 0 || a->batch < 0 || a->num_q_heads <= 0)
         return fail(FDK_ESHAPE, "bad dims R=%d B=%d Hq=%d", a->num_ranks, a->batch, a->num_q_heads);
     if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
@@ -668,16 +736,24 @@ int fdk_probe_linear_read(const void* buf, size_t bytes, int nontemporal, int wo
     if (!aligned16(buf)) return fail(FDK_EALIGN, "buf must be 16-byte aligned");
     if (bytes < 65536) return fail(FDK_ESHAPE, "bytes %zu: at least 64 KB", bytes);
     if (workgroups <= 0 || workgroups > (1 << 20)) return fail(FDK_ESHAPE, "workgroups %d outside [1, 2^20]", workgroups);
-    int rc = fdk::launch_linear_read(buf, bytes, nontemporal, workgroups, reinterpret_cast<hipStream_t>(hip_stream));
+    // the checksum's (practically never taken) store goes to the library's own scratch, not to the caller's buffer
+    void* sink = nullptr;
+    int rc = static_scratch_of_current_device(&sink);
+    if (rc) return rc;
+    sink = static_cast<unsigned char*>(sink) + kStaticScratchBytes;
+    rc = fdk::launch_linear_read(buf, bytes, nontemporal, workgroups, static_cast<uint32_t*>(sink),
+                                 reinterpret_cast<hipStream_t>(hip_stream));
     if (rc) return fail(rc, "linear read launch failed: %s", hipGetErrorString((hipError_t)rc));
     return FDK_OK;
 }
 
-int fdk_kv_append(const fdk_kv_append_args* a, void* hip_stream) {
+int fdk_kv_append(const fdk_kv_append_args* caller_args, void* hip_stream) {
     g_err[0] = 0;
-    if (!a) return fail(FDK_ENULL, "args is null");
-    if (a->struct_size != sizeof(fdk_kv_append_args))
-        return fail(FDK_EABI, "struct_size %u != %zu", a->struct_size, sizeof(fdk_kv_append_args));
+    if (!caller_args) return fail(FDK_ENULL, "args is null");
+    fdk_kv_append_args local;
+    if (int rc = adopt(caller_args, caller_args->struct_size, sizeof(fdk_kv_append_args), "fdk_kv_append_args", &local))
+        return rc;
+    const fdk_kv_append_args* a = &local;
     if (a->batch < 0 || a->new_tokens < 0) return fail(FDK_ESHAPE, "batch %d / new_tokens %d < 0", a->batch, a->new_tokens);
     if (a->num_q_heads < 0 || a->num_kv_heads <= 0)
         return fail(FDK_ESHAPE, "bad head counts Hq=%d Hkv=%d", a->num_q_heads, a->num_kv_heads);

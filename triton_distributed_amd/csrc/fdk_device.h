@@ -48,7 +48,7 @@ struct SplitParams {
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
-    int32_t* length_feedback;       // single pass only: {min, max of the clamped kv_lens, epoch, batch} goes here
+    int32_t* length_feedback;       // set where this kernel ends the call: {min, max of the clamped kv_lens, epoch, batch} goes here
     int32_t feedback_epoch;
     long long* timeline;            // timeline build only (see the split kernel): eight int64 per wavefront
     int64_t timeline_len;
@@ -123,7 +123,8 @@ int launch_kv_append(const KvAppendParams& p, int qkv_dtype, int kv_dtype, hipSt
 int launch_splitkv_valu(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
 int launch_splitkv_mfma_probe(const SplitParams& p, int kv_dtype, hipStream_t stream);      // head_dim 128
-int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream);
+// (sink: four writable bytes for a checksum that is practically never stored; keeps the loads alive)
+int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, uint32_t* sink, hipStream_t stream);
 int launch_combine(const CombineParams& p, hipStream_t stream);
 int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
 bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);

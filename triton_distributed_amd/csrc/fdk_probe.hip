@@ -53,10 +53,8 @@ int launch_splitkv_mfma_probe(const SplitParams& p, int kv_dtype, hipStream_t st
                                     : launch_pm<FDK_BF16, false, 128, true>(p, stream);
 }
 
-int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, hipStream_t stream) {
+int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, uint32_t* sink, hipStream_t stream) {
     const dim3 grid((unsigned)workgroups), block(256);
-    // the first 16 bytes of the buffer double as the (never written) checksum target
-    uint32_t* sink = reinterpret_cast<uint32_t*>(const_cast<void*>(buf));
     const u32x4_t* p = reinterpret_cast<const u32x4_t*>(buf);
     if (nontemporal) hipLaunchKernelGGL(linear_read_kernel<true>, grid, block, 0, stream, p, bytes / 16, sink);
     else hipLaunchKernelGGL(linear_read_kernel<false>, grid, block, 0, stream, p, bytes / 16, sink);

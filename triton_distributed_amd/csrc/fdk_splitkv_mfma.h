@@ -27,9 +27,6 @@
 #pragma once
 
 #include "fdk_device.h"
-#ifdef FDK_TIMELINE
-#include <stdlib.h>
-#endif
 
 namespace fdk {
 
@@ -46,9 +43,9 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 // wavefront leaves eight int64 at p.timeline[8 * (linear workgroup * wavefronts + wavefront)] - the 100 MHz constant
 // clock at kernel entry, before the first K/V loads of its last piece, after that piece's last tile and after its
 // merge and stores (0 if the wavefront left earlier), then the XCD it ran on, the kv head, the sequence and the
-// linear workgroup index.  In that build the environment variable FDK_TIMELINE_ROTATE_HEADS=r makes workgroup x of a
-// sequence take head block (x + r) mod (head blocks) instead of x (chunk mode and single pass, one q-head tile):
-// which XCD reads which head's rows then changes, the rows themselves do not.
+// linear workgroup index.  In that build p.timeline_rotate = r makes workgroup x of a sequence take head block
+// (x + r) mod (head blocks) instead of x (chunk mode and single pass, one q-head tile): which XCD reads which head's
+// rows then changes, the rows themselves do not.
 #ifdef FDK_TIMELINE
 #define FDK_STAMP(i) ts[i] = (long long)__builtin_amdgcn_s_memrealtime()
 #else
@@ -778,6 +775,9 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
         return;
     }
+    // length feedback where this kernel is the last of the call (the single-launch form: no combine follows)
+    if (p.length_feedback && (blockIdx.x | blockIdx.y | blockIdx.z) == 0 && wave == 0)
+        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
     const int units = p.hg_blocks * p.head_tiles;
     // A sequence counts for its granules plus p.piece_cost more in front of them (none if it is empty): every
     // sequence a share begins costs its workgroup a fixed time (table and q loads before the first rows, the merge
@@ -939,12 +939,6 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     // workgroup and register buffers per wavefront (below) follow from the tile size; blocks of 4 or 8 kv heads
     // always take 8 wavefronts.  Measured, batch 32 x 8 kv heads x 4096 tokens: 16-bit cache 85.3 us with two
     // buffers, 81.7 us with one; fp8 cache 52.3 us with 4 wavefronts x 2 buffers, 47.1 us with 8 x 1.
-#ifdef FDK_TIMELINE
-    {
-        const char* rot = getenv("FDK_TIMELINE_ROTATE_HEADS");
-        p.timeline_rotate = rot ? atoi(rot) & 1023 : 0;
-    }
-#endif
     constexpr int kTileBytes = 2 * kTile * D * (FP8 ? 1 : 2);                    // K and V rows of one tile
     const int64_t items = (int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles;
     const bool single_pass = p.num_splits == 1 && !p.balanced;

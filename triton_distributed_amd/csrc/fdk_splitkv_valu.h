@@ -92,6 +92,10 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
     const int head0 = kvh * p.group + ht * GT;      // first q head of this lane
     const int heads_here = min(GT, p.group - ht * GT);
 
+    // length feedback (set only where this kernel is the last of the call: a single pass)
+    if (p.length_feedback && blockIdx.x == 0 && wave == 0)
+        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
+
     const int kv_len = min(p.kv_lens[b], p.max_tokens);
     const int c_start = split * p.chunk;
     if (c_start >= kv_len) {

@@ -40,7 +40,7 @@ from typing import Optional, Sequence, Tuple, Union
 import torch
 
 from . import _lib
-from ._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkPlan
+from ._lib import FdkCombineRanksArgs, FdkDecodeArgs, FdkKvAppendArgs, FdkMeasureArgs, FdkPlan
 
 _LIB = _lib.load()          # raises ImportError when libfdk.so is not built - by design
 
@@ -324,7 +324,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
                    probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0,
                    length_feedback: Optional[LengthFeedback] = None, timeline: Optional[torch.Tensor] = None,
-                   _planned=None) -> PreparedDecode:
+                   rotate_heads=0, _planned=None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -348,7 +348,9 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose.
     ``length_feedback``: a ``LengthFeedback`` that the call's last kernel fills (see there).
     ``timeline``: an int64 GPU tensor, eight values per wavefront of the split kernel; only a library built with
-    ``--timeline`` writes it (``fdk_decode_args.timeline``)."""
+    ``--timeline`` writes it; ``rotate_heads`` moves the head blocks over the workgroups in that build.
+    The measurement aids travel in a ``fdk_measure_args`` block (include/fdk_measure.h) that the argument block points
+    to; a call that uses none of them passes a null pointer, as a product caller does."""
     if not isinstance(kv_lens, torch.Tensor):
         kv_lens = torch.as_tensor(list(kv_lens), dtype=torch.int32, device=q.device)
     # (_planned: the argument block and plan of exactly these arguments, from a caller that has just computed them)
@@ -356,18 +358,22 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len, k_scale, v_scale, algo,
         min_kv_len)
     batch, q_heads, d = q.shape
-    a.tune_wavefronts, a.tune_buffers = int(wavefronts), int(buffers)
-    if shares_per_cu:
-        a.tune_shares_per_cu = int(shares_per_cu)
-        plan = _plan_of(a)                       # this one changes the plan (workgroups, workspace)
+    measure = None
+    if wavefronts or buffers or shares_per_cu or probe_loads or rotate_heads or timeline is not None:
+        measure = FdkMeasureArgs()
+        measure.struct_size = C.sizeof(FdkMeasureArgs)
+        measure.probe_loads = 1 if probe_loads else 0
+        measure.wavefronts, measure.buffers, measure.shares_per_cu = int(wavefronts), int(buffers), int(shares_per_cu)
+        measure.rotate_heads = int(rotate_heads)
+        if timeline is not None:
+            if timeline.dtype != torch.int64 or not timeline.is_cuda or not timeline.is_contiguous():
+                raise ValueError("timeline must be a contiguous int64 GPU tensor")
+            measure.timeline, measure.timeline_len = timeline.data_ptr(), timeline.numel()
+        a.measure = C.addressof(measure)
+        if shares_per_cu:
+            plan = _plan_of(a)                   # this one changes the plan (workgroups, workspace)
     if length_feedback is not None:
         a.length_feedback = length_feedback.device_ptr
-    if timeline is not None:
-        if timeline.dtype != torch.int64 or not timeline.is_cuda or not timeline.is_contiguous():
-            raise ValueError("timeline must be a contiguous int64 GPU tensor")
-        a.timeline, a.timeline_len = timeline.data_ptr(), timeline.numel()
-    if probe_loads:
-        a.flags |= _lib.FDK_FLAG_PROBE_LOADS
     if packed_out is not None:
         if tuple(packed_out.shape) != (batch, q_heads, d + 1) or packed_out.stride(-1) != 1:
             raise ValueError(f"packed output must be [B, Hq, D+1] = {(batch, q_heads, d + 1)}")
@@ -420,7 +426,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         a.counters_len = counters.numel()
     else:
         counters = None
-    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, timeline, counters)
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, timeline, counters,
+            measure)
     return PreparedDecode(a, plan, keep, target, lse)
 
 
