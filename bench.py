@@ -33,9 +33,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=-1,
-                    help="untimed warm-up steps (default: at least 100 and at least 0.1 s of calls - the GPU clock needs some "
-                         "tens of milliseconds of load to come up after the idle time of the input generation, which "
-                         "kernels with much arithmetic per byte (fp8 cache) feel)")
+                    help="untimed warm-up steps; never fewer than 100 calls and 0.1 s of them are run - the GPU clock needs "
+                         "some tens of milliseconds of load to come up after the idle time of the input generation (the "
+                         "JSON line reports the number run as warmup and the number asked for as warmup_requested)")
     ap.add_argument("--config", default="llama3_8b_b32")
     ap.add_argument("--rotate", type=int, default=2,
                     help="distinct KV pools cycled through, so the working set exceeds the 256 MB memory-side cache "
@@ -66,6 +66,16 @@ def parse_args():
                     help="where the K pool and the V pool of a call lie: staggered (default) = one allocation, the V pool "
                          "256 bytes off the K pool modulo 512, as this package's PagedKVCache allocates them "
                          "(triton_distributed_amd.alloc_kv_pools); separate = two independent torch allocations")
+    ap.add_argument("--fp8-fold", action="store_true",
+                    help="fp8 cache: apply the K scale to the logits instead of to every K value "
+                         "(FDK_FLAG_FP8_FOLD_K_SCALE; off the dequantise-then-decode definition by the 16-bit rounding of K)")
+    ap.add_argument("--kernel-only", action="store_true",
+                    help="time the prepared calls only: no legs on other pools, no graph replay, no un-prepared or "
+                         "reference-named entry points, no CPU baseline - for profiler runs, so that every dispatch of a "
+                         "kernel name in the trace belongs to the one plan and the one algorithm that was asked for")
+    ap.add_argument("--batches", type=int, default=5,
+                    help="the K timed steps are run this many times, each bracketed by synchronisations; the median "
+                         "batch is reported (all of them are listed)")
     ap.add_argument("--no-separate-leg", action="store_true",
                     help="do not also time the calls on independently allocated pools (separate_pools_us_per_call); for "
                          "profiler runs, whose per-kernel averages should cover one placement only")
@@ -73,13 +83,21 @@ def parse_args():
     ap.add_argument("--rotate-heads", type=int, default=0, metavar="R",
                     help="--op timeline: workgroup x of a sequence takes head block (x + R) mod (head blocks) - the same rows "
                          "are then read from other XCDs")
-    ap.add_argument("--op", default="decode", choices=["decode", "kv_append", "ceiling", "timeline"],
+    ap.add_argument("--sweep-max-gb", type=float, default=6.0,
+                    help="--op plan-sweep: skip cells whose KV cache exceeds this many GB (they stream for milliseconds and "
+                         "every plan is a single pass)")
+    ap.add_argument("--sweep-heads", default="32/8,64/8,8/1", help="--op plan-sweep: q/kv head pairs")
+    ap.add_argument("--sweep-batches", default="1,4,8,16,24,32,40,64,128")
+    ap.add_argument("--sweep-lens", default="1024,4096,16384,65536")
+    ap.add_argument("--op", default="decode", choices=["decode", "kv_append", "ceiling", "timeline", "plan-sweep"],
                     help="decode: the hot path (default); kv_append: the step before it (RMSNorm + rotary + "
                          "paged append of one new token per sequence) at the same shape; ceiling: what the memory "
                          "system delivers for this configuration with no arithmetic in the way (a streaming read "
                          "of as many bytes, and the split kernel reduced to its load pipeline) next to the kernel; "
                          "timeline: when the wavefronts of the split kernel start, issue their first loads and finish, by "
-                         "XCD and by kv head (needs the measurement build: python -m triton_distributed_amd.build --timeline)")
+                         "XCD and by kv head (needs the measurement build: python -m triton_distributed_amd.build --timeline); "
+                         "plan-sweep: the library's plan against the plans it rejects (single pass, forced split counts, "
+                         "equal shares) over a grid of batch sizes, lengths and head layouts, as a markdown table")
     return ap.parse_args()
 
 
@@ -246,7 +264,8 @@ def bench_ceiling(args):
                                                                dtype=inp.k_cache.dtype))
     pools = _placed(args, tda, [(inp.k_cache, inp.v_cache), (mk(), mk())])
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, always_workspace=True,
-              wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
+              wavefronts=args.wavefronts, buffers=args.buffers, shares_per_cu=args.shares_per_cu,
+              fp8_fold_k_scale=args.fp8_fold, **_hints_of(args, inp))
     real = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, **kw) for k, v in pools]
     probe = [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, probe_loads=True, **kw)
              for k, v in pools]
@@ -365,6 +384,108 @@ def bench_timeline(args):
                       "launches": launches}))
 
 
+def bench_plan_sweep(args):
+    """The plan the library chooses against the alternatives it rejects, cell by cell: bf16, head_dim 128, page size
+    16, batch x length x (q heads / kv heads), in three modes - lengths uniform and known to the host (hinted), uniform
+    and unknown (the table is exactly as wide as the sequences, nothing else is said), and ragged (uniform in
+    [1, N], unknown).  Every plan is timed as a whole call (split kernel + combine) with HIP events around
+    back-to-back launches on one prepared call.  Prints a markdown table and, last, one JSON line with the summary."""
+    import torch
+    import triton_distributed_amd as tda
+
+    dev = torch.device("cuda:0")
+    d, page = 128, 16
+    heads = [tuple(int(x) for x in h.split("/")) for h in args.sweep_heads.split(",")]
+    batches = [int(x) for x in args.sweep_batches.split(",")]
+    lens_list = [int(x) for x in args.sweep_lens.split(",")]
+    cap_bytes = args.sweep_max_gb * 1e9
+    gen = torch.Generator(device=dev).manual_seed(4711)
+
+    def time_call(calls):
+        """(calls: the same plan on distinct regions of the pool, cycled through so that a small cell does not run out
+        of the 256 MB memory-side cache)"""
+        state = {"i": 0}
+
+        class call:
+            @staticmethod
+            def run():
+                calls[state["i"] % len(calls)].run()
+                state["i"] += 1
+        for _ in range(3):
+            call.run()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):                          # best of three short batches: a cell takes milliseconds
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            n = 0
+            t0 = time.perf_counter()
+            e0.record()
+            while n < 5 or (n < 40 and time.perf_counter() - t0 < 1.5e-3):
+                call.run()
+                n += 1
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / n
+            best = us if best is None else min(best, us)
+        return best
+
+    print("| heads | batch | kv_len | mode | library's plan | us | best alternative | us | library / best |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    cells = []
+    for hq, hkv in heads:
+        fits = [(b, n) for b in batches for n in lens_list if b * n * hkv * 2 * d * 2 <= cap_bytes]
+        if not fits:
+            continue
+        max_pages = max(b * n for b, n in fits) // page
+        k, v = tda.alloc_kv_pools((max_pages, page, hkv, d), torch.bfloat16, dev, zero=False)
+        k.normal_(generator=gen)
+        v.normal_(generator=gen)
+        q_all = torch.randn(max(batches), hq, d, generator=gen, device=dev, dtype=torch.bfloat16)
+        for b, n in fits:
+            q = q_all[:b]
+            cell_pages = b * n // page
+            n_rot = max(1, min(8, max_pages // cell_pages, int(1.5e9 // (cell_pages * page * hkv * 2 * d * 2)) + 1))
+            tables = [(torch.randperm(cell_pages, generator=gen, device=dev).to(torch.int32) + r * cell_pages).view(b, n // page)
+                      for r in range(n_rot)]
+            host_gen = torch.Generator().manual_seed(b * 131 + n)
+            modes = [("hinted", torch.full((b,), n, dtype=torch.int32), dict(max_kv_len=n, min_kv_len=n)),
+                     ("unhinted", torch.full((b,), n, dtype=torch.int32), {})]
+            if b > 1:
+                modes.append(("ragged", torch.randint(1, n + 1, (b,), generator=host_gen).to(torch.int32), {}))
+            for mode, lens_host, hints in modes:
+                lens = lens_host.to(dev)
+                alg_bytes = int(lens_host.sum()) * hkv * 2 * d * 2
+                variants = [("library", {})]
+                variants.append(("single pass", dict(kv_split=1)))
+                variants += [(f"{s_} chunks", dict(kv_split=s_)) for s_ in (2, 4, 8, 16, 32) if n // s_ >= 64]
+                if b > 1:
+                    variants.append(("equal shares", dict(force_balanced=True)))
+                res = []
+                for name, kw in variants:
+                    rot = [tda.prepare_decode(q, k, v, t, lens, d ** -0.5, work_queue=False, **hints, **kw) for t in tables]
+                    pl = rot[0].plan
+                    desc = ("single pass" if pl.num_splits == 1 else
+                            f"equal shares, {pl.workgroups} workgroups" if pl.balanced else
+                            f"{pl.num_splits} chunks" + (" of own length" if pl.chunk_floor else "")) + f", {pl.kv_heads_per_wg} kv heads/wg"
+                    res.append((name, desc, time_call(rot)))
+                lib = res[0]
+                best = min(res[1:], key=lambda r: r[2])
+                ratio = lib[2] / best[2]
+                cells.append(dict(heads=f"{hq}/{hkv}", batch=b, kv_len=n, mode=mode, library_plan=lib[1], library_us=round(lib[2], 2),
+                                  best=best[0], best_plan=best[1], best_us=round(best[2], 2), ratio=round(ratio, 3),
+                                  pct_of_peak=round(alg_bytes / lib[2] / 1e3 / HBM_PEAK_GBPS * 100, 1),
+                                  all={r[0]: round(r[2], 2) for r in res}))
+                print(f"| {hq}/{hkv} | {b} | {n} | {mode} | {lib[1]} | {lib[2]:.1f} | {best[0]} ({best[1]}) | {best[2]:.1f} | "
+                      f"{ratio:.3f} |", flush=True)
+        del k, v
+        torch.cuda.empty_cache()
+    worst = sorted(cells, key=lambda c: -c["ratio"])[:12]
+    print()
+    print(json.dumps({"op": "plan-sweep", "cells": len(cells),
+                      "cells_within_5pct_of_best": sum(c["ratio"] <= 1.05 for c in cells),
+                      "worst": worst}), flush=True)
+
+
 def main():
     args = parse_args()
     if args.op == "timeline" and "FDK_LIBRARY" not in os.environ:
@@ -389,6 +510,8 @@ def main():
         return bench_ceiling(args)
     if args.op == "timeline":
         return bench_timeline(args)
+    if args.op == "plan-sweep":
+        return bench_plan_sweep(args)
     t_gen = time.perf_counter()
     inp_cpu = wl.make_inputs(_config_of(args, wl))
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
@@ -411,30 +534,44 @@ def main():
         return [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                    v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
                                    single_launch=args.single_launch, wavefronts=args.wavefronts, buffers=args.buffers,
-                                   shares_per_cu=args.shares_per_cu, **_hints_of(args, inp))
+                                   shares_per_cu=args.shares_per_cu, fp8_fold_k_scale=args.fp8_fold, **_hints_of(args, inp))
                 for k, v in pp]
 
     # ---- the calls on independently allocated pools (the other placement), for the record: timed first, then the
     # pools move into their placed allocations one by one and the originals go back to the driver.  (Freed device
     # memory is wiped in the background, which takes bandwidth for some milliseconds: hence before everything else,
     # followed by a pause, and not in between the timed legs.)
-    separate_us = None
+    separate_us = bare_us = None
+
+    def timed_loop(fn, n):
+        """Wall-clock microseconds per call of n back-to-back fn(i), after at least 100 calls and 0.1 s of them."""
+        n_warm = 0
+        t0 = time.perf_counter()
+        while n_warm < 100 or time.perf_counter() - t0 < 0.1:
+            fn(n_warm)
+            n_warm += 1
+            if n_warm % 50 == 0:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / n
+
+    if args.kernel_only:
+        args.no_separate_leg = args.no_graph = args.no_cpu_baseline = True
+    if not args.no_separate_leg and not args.kernel_only:
+        # the bare signature of the path, flash_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale) and nothing
+        # else - no length bounds, no placement of the pools, outputs and scratch left to the call - on independently
+        # allocated pools: what a caller that knows only the reference's interface gets
+        kw_bare = dict(k_scale=inp.k_scale, v_scale=inp.v_scale) if inp.cfg.kv_dtype == "fp8_e4m3" else {}
+        bare_us = timed_loop(lambda i: tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens,
+                                                        inp.sm_scale, **kw_bare), args.steps)
     if args.kv_placement == "staggered":
         if not args.no_separate_leg:
             sep = prepare_all(pools)
-            n_warm = 0
-            t0 = time.perf_counter()
-            while n_warm < 100 or time.perf_counter() - t0 < 0.1:
-                sep[n_warm % len(sep)].run()
-                n_warm += 1
-                if n_warm % 50 == 0:
-                    torch.cuda.synchronize()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for i in range(args.steps):
-                sep[i % len(sep)].run()
-            torch.cuda.synchronize()
-            separate_us = (time.perf_counter() - t0) * 1e6 / args.steps
+            separate_us = timed_loop(lambda i: sep[i % len(sep)].run(), args.steps)
             del sep
         placed = []
         while pools:
@@ -466,44 +603,56 @@ def main():
     def step(i):
         calls[i % len(calls)].run()
 
-    # ---- whole call: W warm-up, then exactly K timed steps ----------------------------------------------------
-    if args.warmup < 0:
-        for i in range(10):
-            step(i)
+    # ---- whole call: W warm-up steps (never fewer than 100 calls and 0.1 s of them: after the idle seconds of the
+    # input generation the GPU clock needs some tens of milliseconds of load to come up, and a handful of calls does
+    # not give it that), then exactly K timed steps between synchronisations - `--batches` times over, the median
+    # batch being the one reported.  HIP events on the launch stream go around the same K steps: for a single-pass
+    # plan the call IS one launch of the split kernel, so the events give that kernel's average duration over the very
+    # launches the wall clock timed (events sit inside the synchronisations, hence us_per_launch <= us_per_call).
+    single_pass = plan.num_splits == 1
+    requested_warmup = args.warmup
+    n_warm = 0
+    t0 = time.perf_counter()
+    while n_warm < max(args.warmup, 100) or time.perf_counter() - t0 < 0.1:
+        step(n_warm)
+        n_warm += 1
+        if n_warm % 50 == 0:
+            torch.cuda.synchronize()
+    args.warmup = n_warm
+    batches = []
+    for _ in range(max(1, args.batches)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(20):
+        e0.record()
+        for i in range(args.steps):
             step(i)
+        e1.record()
         torch.cuda.synchronize()
-        per_call = max((time.perf_counter() - t0) / 20, 1e-6)
-        args.warmup = max(100, int(0.1 / per_call))
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    torch.cuda.synchronize()
-    wall_s = time.perf_counter() - t0
+        batches.append(((time.perf_counter() - t0), e0.elapsed_time(e1) * 1e-3))
+    wall_s, events_s = sorted(batches)[len(batches) // 2]
     ms_per_step = wall_s * 1e3 / args.steps
     gbps = alg_bytes / (wall_s / args.steps) / 1e9
 
-    # ---- dominant kernel alone (split-KV), HIP events on the launch stream ------------------------------------
-    # A single-pass plan runs one kernel, the variant that writes (out, lse) itself: the events go around the call.
-    # A split plan runs the split kernel and the combine: the events go around the split launches only.
-    single_pass = plan.num_splits == 1
-    kernel_step = (lambda i: calls[i % len(calls)].run()) if single_pass else \
-        (lambda i: calls[i % len(calls)].run_splitkv())
-    for i in range(min(args.warmup, 10)):
-        kernel_step(i)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    for i in range(args.steps):
-        kernel_step(i)
-    e1.record()
-    torch.cuda.synchronize()
-    split_us = e0.elapsed_time(e1) * 1e3 / args.steps
+    # ---- dominant kernel alone (split-KV).  Single pass: the events of the timed loop above.  A split plan runs the
+    # split kernel and the combine: events go around launches of the split kernel only, warmed up like the call.
+    if single_pass:
+        split_us = events_s * 1e6 / args.steps
+    else:
+        kernel_step = lambda i: calls[i % len(calls)].run_splitkv()
+        for i in range(100):
+            kernel_step(i)
+        reps = []
+        for _ in range(max(1, args.batches)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(args.steps):
+                kernel_step(i)
+            e1.record()
+            torch.cuda.synchronize()
+            reps.append(e0.elapsed_time(e1) * 1e3 / args.steps)
+        split_us = sorted(reps)[len(reps) // 2]
     split_gbps = alg_bytes / (split_us * 1e-6) / 1e9
 
     # ---- the same calls replayed from one HIP graph (a serving engine replays its decode step from a graph):
@@ -536,31 +685,20 @@ def main():
 
     # ---- the un-prepared public entry point: flash_decode() validates, marshals and allocates (out, lse) per call
     kw = dict(k_scale=inp.k_scale, v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, **_hints_of(args, inp))
-    n_entry = min(args.steps, 100)
-    for i in range(5):
-        tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens, inp.sm_scale, **kw)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(n_entry):
-        tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens, inp.sm_scale, **kw)
-    torch.cuda.synchronize()
-    entry_us = (time.perf_counter() - t0) * 1e6 / n_entry
+    n_entry = max(args.steps, 100)
+    entry_us = None
+    if not args.kernel_only:
+        entry_us = timed_loop(lambda i: tda.flash_decode(inp.q, *pools[i % len(pools)], inp.block_table, inp.kv_lens,
+                                                         inp.sm_scale, **kw), n_entry)
 
     # ---- the drop-in for the reference's entry point, called the way the reference's layer calls it: no length bounds,
     # kv_split = 32 (sp_flash_decode_layer.py:62,100-110), output_combine given; fp8 caches are not part of that signature
-    ref_entry_us = ref_entry_fb_us = None
-    if inp.cfg.kv_dtype != "fp8_e4m3":
+    ref_entry_us = ref_entry_fb_us = cold_fb_us = None
+    if inp.cfg.kv_dtype != "fp8_e4m3" and not args.kernel_only:
         oc = torch.empty((inp.q.shape[0], inp.q.shape[1], inp.q.shape[2] + 1), dtype=inp.q.dtype, device=dev)
         ref_call = lambda i: tda.gqa_fwd_batch_decode_intra_rank(inp.q, *pools[i % len(pools)], None, None, inp.kv_lens,
                                                                  inp.block_table, inp.sm_scale, output_combine=oc, kv_split=32)
-        for i in range(5):
-            ref_call(i)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(n_entry):
-            ref_call(i)
-        torch.cuda.synchronize()
-        ref_entry_us = (time.perf_counter() - t0) * 1e6 / n_entry
+        ref_entry_us = timed_loop(ref_call, n_entry)
         # the same entry point with a LengthFeedback block, as the layer mirror keeps one: each call plans with the
         # bounds of kv_lens that the previous call's last kernel left in pinned host memory
         fb = tda.LengthFeedback()
@@ -570,11 +708,25 @@ def main():
         for i in range(5):
             fb_call(i)
             torch.cuda.synchronize()
+        ref_entry_fb_us = timed_loop(fb_call, n_entry)
+        # ... and what the FIRST call on a feedback block costs (a new batch, a new layer object): every call of this
+        # loop is given a block that no call has written yet, so it plans for unknown lengths and only leaves bounds
+        cold = [tda.LengthFeedback() for _ in range(n_entry + 128)]
+        n_cold = iter(range(len(cold)))
+        cold_call = lambda i: tda.gqa_fwd_batch_decode_intra_rank(inp.q, *pools[i % len(pools)], None, None, inp.kv_lens,
+                                                                  inp.block_table, inp.sm_scale, output_combine=oc,
+                                                                  kv_split=32, length_feedback=cold[next(n_cold)])
+        for i in range(100):                       # warm-up on blocks of their own
+            cold_call(i)
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(n_entry):
-            fb_call(i)
+            cold_call(i)
         torch.cuda.synchronize()
-        ref_entry_fb_us = (time.perf_counter() - t0) * 1e6 / n_entry
+        cold_fb_us = (time.perf_counter() - t0) * 1e6 / n_entry
+        assert all(c.read()[2] != 0 for c in cold[:n_entry + 100])        # every block was written exactly by its call
+        for c in cold:
+            c.close()
 
     traffic = None
     traffic_source = None
@@ -595,14 +747,19 @@ def main():
         "unit": "GB/s",
         "us_per_call": round(ms_per_step * 1e3, 2),
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "batches_us_per_call": [round(w * 1e6 / args.steps, 2) for w, _ in batches],
+        "no_hints_us_per_call": None if bare_us is None else round(bare_us, 2),
+        "no_hints_pct_of_hbm_peak": None if bare_us is None else round(alg_bytes / bare_us / 1e3 / HBM_PEAK_GBPS * 100, 2),
         "separate_pools_us_per_call": None if separate_us is None else round(separate_us, 2),
         "graph_replay_us_per_call": None if graph_us is None else round(graph_us, 2),
-        "public_entry_us_per_call": round(entry_us, 2),
+        "public_entry_us_per_call": None if entry_us is None else round(entry_us, 2),
         "reference_entry_us_per_call": None if ref_entry_us is None else round(ref_entry_us, 2),
         "reference_entry_with_feedback_us_per_call": None if ref_entry_fb_us is None else round(ref_entry_fb_us, 2),
+        "first_call_with_cold_feedback_us": None if cold_fb_us is None else round(cold_fb_us, 2),
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_requested": requested_warmup,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -618,6 +775,8 @@ def main():
             "algo": plan.algo,
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "single_launch": bool(args.single_launch and plan.num_splits > 1),
+            "fp8_k_scale": None if inp.cfg.kv_dtype != "fp8_e4m3" else
+                           ("folded into the logit scale" if args.fp8_fold else "applied to every K value (exact dequantisation)"),
             "kv_pool_placement": ("one allocation per (K, V) pair, V 256 bytes off K modulo 512 (alloc_kv_pools, as PagedKVCache "
                                   "allocates)" if args.kv_placement == "staggered" else "two independent torch allocations"),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,
@@ -634,6 +793,8 @@ def main():
             "unit": "GB/s",
             "frac": round(split_gbps / HBM_PEAK_GBPS, 4),
             "us_per_launch": round(split_us, 2),
+            "timed": "HIP events around the K timed steps of the reported batch" if single_pass else
+                     "HIP events around K launches of the split kernel alone (median of the batches)",
             "traffic": traffic,
             "traffic_source": traffic_source,
         },

@@ -42,6 +42,12 @@ typedef struct fdk_measure_args {
     int32_t rotate_heads;
     int64_t* timeline;
     int64_t timeline_len;
+
+    /* 1: plan equal shares of the whole batch (balanced mode) wherever the matrix-core path can run them (two or more
+     * sequences), whatever the length hints say - for timing that plan against the one the library chooses
+     * (bench.py --op plan-sweep).  Changes the plan (workgroups, workspace), never results. */
+    int32_t force_balanced;
+    int32_t reserved;
 } fdk_measure_args;
 
 /* A streaming read of buf[0, bytes) by `workgroups` workgroups of 256 threads with 16-byte loads (non-temporal if

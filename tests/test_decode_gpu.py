@@ -1401,6 +1401,66 @@ def test_fp8_kv_cache_small(cuda_device, heads, algo):
     torch.testing.assert_close(lse.double(), l64, atol=5e-3, rtol=0)
 
 
+@pytest.mark.parametrize("heads,page,lens", [((32, 8), 16, (1, 2000)), ((64, 8), 16, (1, 2000)), ((8, 8), 1, (1, 700)),
+                                             ((16, 2), 16, [33000, 100, 8000]), ((8, 1), 16, [1, 2, 17, 64, 65])])
+def test_fp8_folded_k_scale(cuda_device, heads, page, lens):
+    """FDK_FLAG_FP8_FOLD_K_SCALE: logits are (q . k8) * k_scale instead of q . round_bf16(k8 * k_scale).  That is the
+    exact evaluation of what the cache holds: against the float64 attention over k8 * k_scale (no rounding of K) the
+    bars of this path hold as they are (lse 1e-3).  Against the dequantise-to-bf16-then-decode definition - the oracle
+    of the default form - single logits differ by the 16-bit rounding of K (about 1e-3 for 128 unit-variance terms),
+    so lse is compared at 5e-3 there, out at the usual 2e-2; short and peaked sequences are where the two definitions
+    are furthest apart, long diffuse ones agree to 1e-4 (the benchmark configuration is checked at the standard bars in
+    test_config5_fp8_70b_b128_folded_k_scale)."""
+    g = torch.Generator().manual_seed(91 + heads[0] + page)
+    if isinstance(lens, tuple):
+        lens = torch.randint(lens[0], lens[1] + 1, (5,), generator=g).tolist()
+    hq, hkv, d = heads[0], heads[1], 128
+    pages = [(n + page - 1) // page for n in lens]
+    pool = sum(pages) + 3
+    table = torch.full((len(lens), max(pages) + 2), 2 ** 31 - 1, dtype=torch.int32)      # poisoned beyond each sequence
+    perm = torch.randperm(pool, generator=g).to(torch.int32)
+    at = 0
+    for i, n in enumerate(pages):
+        table[i, :n] = perm[at:at + n]
+        at += n
+    k8, ks = wl.quantize_kv_fp8(torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device))
+    v8, vs = wl.quantize_kv_fp8(torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device))
+
+    class inp:                                          # the names the checks below use
+        q = torch.randn(len(lens), hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+        k_cache, v_cache, k_scale, v_scale = k8, v8, ks, vs
+        block_table = table.to(cuda_device)
+        kv_lens, kv_lens_host, sm_scale = _lens_t(lens, cuda_device), list(lens), d ** -0.5
+    results = {}
+    for fold in (False, True):
+        for kw in (dict(), dict(kv_split=1), dict(kv_split=5)):
+            out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                        k_scale=inp.k_scale, v_scale=inp.v_scale, fp8_fold_k_scale=fold, **kw)
+            torch.cuda.synchronize()
+            results[(fold, tuple(kw.items()))] = (out.clone(), lse.clone())
+    kd = ofp8.dequant_per_head(inp.k_cache, inp.k_scale)
+    vd = ofp8.dequant_per_head(inp.v_cache, inp.v_scale)
+    ref = ref_paged_attn(inp.q, kd, vd, inp.kv_lens_host, inp.block_table, inp.sm_scale)
+    _, l_deq = cf.attn_fp64(inp.q, kd, vd, inp.block_table, inp.kv_lens_host, inp.sm_scale)
+    o64, l64 = cf.attn_fp64(inp.q, inp.k_cache.float(), inp.v_cache.float(), inp.block_table, inp.kv_lens_host,
+                            inp.sm_scale, k_scale=inp.k_scale, v_scale=inp.v_scale)
+    for (fold, kw), (out, lse) in results.items():
+        assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all(), (fold, kw)
+        torch.testing.assert_close(out.float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL, msg=lambda m: f"fold={fold} {kw}: {m}")
+        if fold:
+            torch.testing.assert_close(lse.double(), l64, atol=LSE_ATOL, rtol=0, msg=lambda m: f"folded vs exact cache {kw}: {m}")
+            torch.testing.assert_close(out.double(), o64, atol=8e-3, rtol=1e-2)
+            torch.testing.assert_close(lse.double(), l_deq, atol=5e-3, rtol=0)
+        else:
+            torch.testing.assert_close(lse.double(), l_deq, atol=LSE_ATOL, rtol=0, msg=lambda m: f"default form {kw}: {m}")
+    # the flag changes nothing for a 16-bit cache
+    k16, v16 = kd.contiguous(), vd.contiguous()
+    a = tda.flash_decode(inp.q, k16, v16, inp.block_table, inp.kv_lens, inp.sm_scale)
+    b = tda.flash_decode(inp.q, k16, v16, inp.block_table, inp.kv_lens, inp.sm_scale, fp8_fold_k_scale=True)
+    torch.cuda.synchronize()
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
 @pytest.mark.parametrize("algo", ["valu", "mfma"])
 def test_fp8_every_byte_value_dequantises_exactly(cuda_device, algo):
     # 254 finite e4m3 codes as single-token V rows: out must equal table[code] * scale bit-exactly in fp32
@@ -1502,6 +1562,15 @@ def test_config4_long_131k(cuda_device, algo):
 def test_config5_fp8_70b_b128(cuda_device, algo):
     inp, out, lse = _full_config("fp8_70b_b128", cuda_device, algo)
     _check_rows(inp, out, lse, range(0, 128, 9) if algo == "auto" else [5, 100], "cfg5")
+
+
+def test_config5_fp8_70b_b128_folded_k_scale(cuda_device):
+    # the folded form of the fp8 K scale against the SAME oracle and bars as the default form (dequantise to bf16, then
+    # decode: out 2e-2, lse 1e-3): 8192 tokens per sequence average the 16-bit rounding of K away
+    cfg = wl.CONFIGS["fp8_70b_b128"]
+    for hints in (dict(), dict(max_kv_len=cfg.kv_len, min_kv_len=cfg.kv_len)):
+        inp, out, lse = _full_config("fp8_70b_b128", cuda_device, fp8_fold_k_scale=True, **hints)
+        _check_rows(inp, out, lse, range(0, 128, 13), f"cfg5 folded {hints}")
 
 
 def test_config5_fp8_70b_b128_with_the_length_hints_of_the_benchmark(cuda_device):
@@ -1643,3 +1712,88 @@ def test_load_only_probes_run_and_leave_the_inputs_alone(cuda_device):
     out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale)
     torch.cuda.synchronize()
     _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale, tag="after probe")
+
+
+def test_shared_scratch_of_a_foreign_stream_is_not_reused_by_the_current_one(cuda_device):
+    # flash_decode(..., stream=side) keeps its split partials in a buffer shared by the calls of that stream and grows
+    # it on demand.  The buffer belongs to the side stream's memory pool: while the side stream's kernels still write
+    # partial rows, the default stream allocates and fills tensors of the very sizes that were just dropped - they must
+    # never be handed the memory of a buffer that is still in use.
+    side = torch.cuda.Stream(device=cuda_device)
+    cases = []
+    for i, (b, n) in enumerate([(1, 3000), (2, 9000), (3, 20000), (5, 40000)]):       # growing workspaces
+        inp = wl.make_inputs(wl.scaled_down(wl.CONFIGS["ragged_g8"], batch=b, kv_len_range=(n // 2, n)), cuda_device)
+        plan = tda.get_split_kv_plan(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens)
+        assert plan.num_splits > 1, (b, n)
+        cases.append((inp, plan.workspace_bytes))
+    assert [w for _, w in cases] == sorted(w for _, w in cases) and cases[0][1] < cases[-1][1]
+    torch.cuda.synchronize()
+    results, hogs = [], []
+    side.wait_stream(torch.cuda.current_stream())
+    for rep in range(3):
+        for inp, ws in cases:
+            out, lse = tda.flash_decode(inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens, inp.sm_scale,
+                                        stream=side)
+            results.append((inp, out, lse))
+            # the default stream, unsynchronised with the side stream: same-sized allocations, filled at once
+            for nbytes in {w for _, w in cases}:
+                hogs.append(torch.full((nbytes,), 0x7f, dtype=torch.uint8, device=cuda_device))
+            hogs = hogs[-8:]
+        import importlib
+        fd = importlib.import_module("triton_distributed_amd.flash_decode")
+        fd._SCRATCH_CACHE.clear()                  # the next round grows the buffer again from the smallest size
+    side.synchronize()
+    torch.cuda.synchronize()
+    for i, (inp, out, lse) in enumerate(results):
+        _check(out, lse, inp.q, inp.k_cache, inp.v_cache, inp.block_table, inp.kv_lens_host, inp.sm_scale,
+               tag=f"foreign stream call {i}")
+
+
+def test_captured_drop_in_call_with_feedback_follows_grown_lengths(cuda_device):
+    # A drop-in entry point that is given a LengthFeedback block plans with the bounds the previous call left there -
+    # but not while its stream is capturing: a graph is replayed while kv_lens grows, and bounds baked into it (here
+    # about 500 tokens) would size the chunks of every replay, the last chunk taking all the rest.  Capture at N,
+    # replay at about 8 N: right result, and no slower than a few times the eager call planned for that length.
+    import time
+    b, hq, hkv, d, page, n0, n1 = 4, 32, 8, 128, 16, 500, 4000
+    g = torch.Generator().manual_seed(77)
+    pages = (n1 + page - 1) // page
+    pool = b * pages
+    q = torch.randn(b, hq, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    k = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    v = torch.randn(pool, page, hkv, d, generator=g).to(torch.bfloat16).to(cuda_device)
+    table = torch.randperm(pool, generator=g).to(torch.int32).view(b, pages).to(cuda_device)
+    lens = torch.full((b,), n0, dtype=torch.int32, device=cuda_device)
+    fb = tda.LengthFeedback()
+    oc = torch.empty(b, hq, d + 1, dtype=torch.bfloat16, device=cuda_device)
+    call = lambda: tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, None, lens, table, d ** -0.5, output_combine=oc,
+                                                       kv_split=32, length_feedback=fb)
+    for _ in range(3):                                  # eager warm-up: the block now holds (n0, n0)
+        call()
+        torch.cuda.synchronize()
+    assert fb.bounds(b) == (n0, n0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    lens.fill_(n1)
+    oc.fill_(float("nan"))
+    graph.replay()
+    torch.cuda.synchronize()
+    assert fb.bounds(b) == (n1, n1)                     # the replay still reports what it ran on
+    out, lse = oc[..., :d].clone(), oc[..., d].float().clone()
+    ref = ref_paged_attn(q, k, v, [n1] * b, table, d ** -0.5)
+    torch.testing.assert_close(out.float(), ref.float(), atol=OUT_ATOL, rtol=OUT_RTOL)
+    _, l64 = cf.attn_fp64(q, k, v, table, [n1] * b, d ** -0.5)
+    torch.testing.assert_close(lse.double(), l64, atol=5e-2, rtol=1e-2)      # lse went through bf16 in the packed row
+
+    def timed(fn, n=20):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+    t_graph = timed(graph.replay)
+    t_eager = timed(lambda: tda.flash_decode(q, k, v, table, lens, d ** -0.5, max_kv_len=n1, min_kv_len=n1))
+    assert t_graph < 4 * t_eager + 50e-6, (t_graph, t_eager)

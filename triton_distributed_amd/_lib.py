@@ -21,7 +21,7 @@ FDK_OK, FDK_ENULL, FDK_EALIGN, FDK_ESHAPE, FDK_EUNSUPPORTED, FDK_EWORKSPACE, FDK
 # fdk_algo
 FDK_ALGO_AUTO, FDK_ALGO_VALU, FDK_ALGO_MFMA = 0, 1, 2
 # flags
-FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_SINGLE_LAUNCH = 1, 2, 8
+FDK_FLAG_PACK_LSE, FDK_FLAG_DRY_RUN, FDK_FLAG_SINGLE_LAUNCH, FDK_FLAG_FP8_FOLD_K_SCALE = 1, 2, 8, 16
 FDK_STATIC_SCRATCH_BYTES = 32 << 20
 
 # declared in include/fdk.h
@@ -71,6 +71,7 @@ class FdkMeasureArgs(C.Structure):
         ("struct_size", C.c_uint32), ("probe_loads", C.c_uint32),
         ("wavefronts", C.c_int32), ("buffers", C.c_int32), ("shares_per_cu", C.c_int32), ("rotate_heads", C.c_int32),
         ("timeline", C.c_void_p), ("timeline_len", C.c_int64),
+        ("force_balanced", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

@@ -176,6 +176,8 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         if (m->shares_per_cu < 0 || m->shares_per_cu > 4)
             return fail(FDK_ESHAPE, "measure: shares_per_cu %d (0 .. 4)", m->shares_per_cu);
         if (m->probe_loads > 1) return fail(FDK_ESHAPE, "measure: probe_loads %u (0, 1)", m->probe_loads);
+        if (m->force_balanced < 0 || m->force_balanced > 1)
+            return fail(FDK_ESHAPE, "measure: force_balanced %d (0, 1)", m->force_balanced);
         if (m->timeline && ((reinterpret_cast<uintptr_t>(m->timeline) & 7u) || m->timeline_len < 0))
             return fail(FDK_EALIGN, "measure: timeline must be 8-byte aligned, timeline_len >= 0");
     }
@@ -281,8 +283,13 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * 2.0 * a->head_dim *
                              elem_size(a->kv_dtype) / kStreamBytesPerUs;      // what streaming the batch's cache takes
     bool rebalance = false;
+    // (measurement aid: equal shares wherever they can run, to time them against the plan chosen here)
+    const bool force_balanced = a->measure && a->measure->force_balanced && algo == FDK_ALGO_MFMA && a->num_splits <= 0 &&
+                                batch > 1 && batch <= kMaxBalancedBatch;
     if (algo == FDK_ALGO_MFMA && a->num_splits <= 0 && units >= num_cus && batch <= kMaxBalancedBatch) {
-        if (!alike) {
+        if (force_balanced) {
+            rebalance = true;
+        } else if (!alike) {
             rebalance = units < 4 * (int64_t)num_cus && max_len >= kMinRaggedLen;
         } else if (units > num_cus) {
             const int64_t rounds = cdiv64(units, num_cus);
@@ -306,7 +313,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     if (min_chunk < kMinChunk) min_chunk = kMinChunk;
     if (min_chunk > kMaxMinChunk) min_chunk = kMaxMinChunk;
     const int64_t most_chunks = cdiv64(max_len, min_chunk);
-    const bool may_split = a->num_splits <= 0 && (units < num_cus || rebalance) && most_chunks > 1;
+    const bool may_split = a->num_splits <= 0 && (units < num_cus || rebalance) && (most_chunks > 1 || force_balanced);
     int64_t splits = 1;
     if (a->num_splits > 0) {
         splits = a->num_splits;
@@ -336,7 +343,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         const double slower = 0.75 * (0.82 - fill);
         underfilled = slower > 0.0 && stream_us * slower > 1.2 * kBalancedExtraUs;
     }
-    const bool uniform = alike && !rebalance && !underfilled;
+    const bool uniform = alike && !rebalance && !underfilled && !force_balanced;
     // (a single sequence has nothing to balance: its own length in equal chunks, below, does the same without the
     // pass over kv_lens and with a combine that knows where its rows are - 27 us against 34 us for 32768 tokens)
     if (algo == FDK_ALGO_MFMA && may_split && !uniform && batch > 1 && batch <= kMaxBalancedBatch &&
@@ -353,7 +360,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         const int64_t share_tokens = cdiv64(columns, shares) * gran;
         // Deriving the partition costs every workgroup a pass over kv_lens before its first load: worth it
         // only when a share is long enough to hide that.
-        if (share_tokens >= kMinBalancedShare) {
+        if (share_tokens >= kMinBalancedShare || force_balanced) {
             const int64_t rows_per_slot = (int64_t)kv_heads_per_wg * (group < 16 ? group : 16);
             const int64_t rows = (shares + batch) * units_per_seq * rows_per_slot;
             plan->balanced = 1;
@@ -461,6 +468,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.out_dtype = a->out_dtype;
     sp.pack_lse = (a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0;
     sp.direct = direct ? 1 : 0;
+    sp.fp8_fold = (a->flags & FDK_FLAG_FP8_FOLD_K_SCALE) && a->kv_dtype == FDK_FP8_E4M3 ? 1 : 0;
     // length feedback: stored by the last kernel of the call - a single pass (or the single-launch form) itself,
     // else the combine kernel
     static std::atomic<int32_t> epoch{0};

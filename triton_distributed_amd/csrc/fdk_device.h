@@ -53,6 +53,7 @@ struct SplitParams {
     long long* timeline;            // timeline build only (see the split kernel): eight int64 per wavefront
     int64_t timeline_len;
     int32_t timeline_rotate;        // timeline build only: rotation of the head blocks over the workgroups
+    int32_t fp8_fold;               // fp8 cache, matrix-core path: the K scale multiplies the logits (see the kernel)
     int32_t probe;                  // 1: load pipeline only (measurement aid), no results
     uint32_t ws_bytes;              // fused: bytes of the workspace (part_o onwards), below 2^32
     int32_t fused;                  // 1: the last piece of a (sequence, head block, head tile) to finish merges its

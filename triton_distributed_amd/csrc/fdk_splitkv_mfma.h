@@ -358,6 +358,14 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     }
     const bool softcap = p.soft_cap > 0.f;
     const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
+    // fp8 K, two forms.  Exact (default): every value becomes round_to_q_dtype(k8 * scale) before the product, i.e. the
+    // logits of a decode over the dequantised cache, at two conversions, four multiplications and two packings per
+    // four values.  Folded (p.fp8_fold): the values are converted exactly (two instructions per four values) and the
+    // head's scale multiplies the logits - (q . k8) * scale instead of q . round(k8 * scale), which differs by the
+    // rounding of K to the 16-bit type (relative 2^-9 per element).
+    const bool fold = FP8 && p.fp8_fold;
+    const float logit_scale_log2 = fold ? p.scale_log2 * kscale : p.scale_log2;
+    const float logit_scale = fold ? p.sm_scale * kscale : p.sm_scale;
 
     const char* kbase = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES + lpiece * 16;
     const char* vbase = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES + lpiece * 16;
@@ -447,13 +455,24 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             for (int j = 0; j < NJ; ++j) {
                 const int r = j * RPL + lrow;
                 uint32_t ko[8], vo[8];
+                if (fold) {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        ko[2 * w] = P2::from_fp8(rg.k[j][w], false);
+                        ko[2 * w + 1] = P2::from_fp8(rg.k[j][w], true);
+                    }
+                } else {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        // K: (k8 * scale) rounded to the q dtype, i.e. the dequantised cache the reference decodes
+                        const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], false);
+                        const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], true);
+                        ko[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
+                        ko[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
+                    }
+                }
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    // K: (k8 * scale) rounded to the q dtype, i.e. the dequantised cache the reference decodes
-                    const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], false);
-                    const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(rg.k[j][w], true);
-                    ko[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
-                    ko[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
                     // V: exact conversion; its scale multiplies the output once at the end
                     vo[2 * w] = P2::from_fp8(rg.v[j][w], false);
                     vo[2 * w + 1] = P2::from_fp8(rg.v[j][w], true);
@@ -508,10 +527,10 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         float sv[4] = {s.x, s.y, s.z, s.w};
         if (softcap) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * p.sm_scale, p.soft_cap, inv_cap) * kLog2e;
+            for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * logit_scale, p.soft_cap, inv_cap) * kLog2e;
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) sv[i] *= p.scale_log2;
+            for (int i = 0; i < 4; ++i) sv[i] *= logit_scale_log2;
         }
         if (MASKED) {                         // the partial last tile of the chunk
 #pragma unroll

@@ -190,18 +190,21 @@ def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv
     return a
 
 
-_TEMPLATES = {}          # layout key -> (validated argument block without pointers, its plan)
+_TEMPLATES = {}          # layout key -> [validated argument block without pointers and bounds, {bounds: plan}]
 
 
 def _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len, k_scale, v_scale,
                    algo, min_kv_len):
     """``_fill_args`` + ``_plan_of`` with a cache: a serving loop calls with the same layouts over and over, and the
-    shape checks and the planning depend on shapes, strides, dtypes, devices and scalars only.  A hit copies the
-    validated block and sets the pointers (their alignment is checked by the library on every call)."""
+    shape checks depend on shapes, strides, dtypes, devices and scalars only.  A hit copies the validated block and sets
+    the pointers (their alignment is checked by the library on every call) and the length bounds; the plan is kept per
+    pair of bounds, so a caller whose bounds move with every decode step (``LengthFeedback``) pays one ``fdk_plan``
+    call for them, not the checks."""
     def meta(t):
         return None if t is None else (t.shape, t.stride(), t.dtype, t.device)
     key = (meta(q), meta(k_cache), meta(v_cache), meta(block_table), meta(kv_lens), meta(k_scale), meta(v_scale),
-           sm_scale, soft_cap, kv_split, max_kv_len, min_kv_len, algo)
+           sm_scale, soft_cap, kv_split, algo)
+    bounds = (int(max_kv_len) if max_kv_len else 0, int(min_kv_len) if min_kv_len else 0)
     hit = _TEMPLATES.get(key)
     if hit is None:
         a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
@@ -209,16 +212,23 @@ def _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap
         plan = _plan_of(a)
         if len(_TEMPLATES) >= 256:
             _TEMPLATES.clear()
-        _TEMPLATES[key] = (bytes(a), plan)
+        _TEMPLATES[key] = [bytes(a), {bounds: plan}]
         return a, plan
     a = FdkDecodeArgs.from_buffer_copy(hit[0])
     a.q, a.k_cache, a.v_cache = q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr()
     a.block_table, a.kv_lens = block_table.data_ptr(), kv_lens.data_ptr()
+    a.max_kv_len, a.min_kv_len = bounds
     if k_scale is not None:
         a.k_scale = k_scale.data_ptr()
     if v_scale is not None:
         a.v_scale = v_scale.data_ptr()
-    return a, hit[1]
+    plan = hit[1].get(bounds)
+    if plan is None:
+        plan = _plan_of(a)                      # (also where the library refuses the bounds)
+        if len(hit[1]) >= 64:
+            hit[1].clear()
+        hit[1][bounds] = plan
+    return a, plan
 
 
 def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
@@ -249,6 +259,32 @@ def _capturing() -> bool:
     return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
 
 
+class _on_stream:
+    """Make the stream with this raw handle torch's current stream while a shared per-stream buffer is (re)allocated.
+
+    torch's caching allocator ties a block to the stream that was current when it was allocated: a block that is freed
+    can be handed out again at once to later work on that stream, and only there.  The shared buffers are used by kernels
+    on the stream whose handle the caller passed, which need not be torch's current one: allocated under the current
+    stream, a buffer that is dropped when a larger one takes its place could be reused by the current stream while
+    kernels on the caller's stream still write partial rows into it (and a fresh zero-fill would not be ordered before
+    its first use).  Allocated under the caller's stream, both the fill and the reuse are ordered with its kernels."""
+
+    def __init__(self, device: torch.device, handle: int):
+        self._ctx = None
+        current = _RAW_STREAM(device.index) if _RAW_STREAM is not None else torch.cuda.current_stream(device).cuda_stream
+        if handle != current:
+            self._ctx = torch.cuda.stream(torch.cuda.ExternalStream(handle, device=device))
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            return self._ctx.__exit__(*exc)
+        return False
+
+
 def _stream_counters(device: torch.device, stream, n: int) -> Optional[torch.Tensor]:
     """Zeroed int32 counters shared by the eager calls issued on one stream (they run in order, and every call
     leaves the counters zero), so the convenience entry points need no fill launch per call.  A call made while
@@ -256,10 +292,12 @@ def _stream_counters(device: torch.device, stream, n: int) -> Optional[torch.Ten
     allocates them): a replay may run on another stream and overlap eager calls on this one."""
     if device.type != "cuda" or _capturing():
         return None                                   # CPU tensors: the caller is about to be told there is no CPU path
-    key = (device.index, _stream_handle(stream))
+    handle = _stream_handle(stream)
+    key = (device.index, handle)
     t = _COUNTER_CACHE.get(key)
     if t is None or t.numel() < n:
-        t = torch.zeros(max(n, 1024), dtype=torch.int32, device=device)
+        with _on_stream(device, handle):
+            t = torch.zeros(max(n, 1024), dtype=torch.int32, device=device)
         _COUNTER_CACHE[key] = t
     return t
 
@@ -269,10 +307,14 @@ def _stream_scratch(device: torch.device, stream, nbytes: int) -> Optional[torch
     demand: calls on one stream run in order, so they can share it.  Not used while capturing (see above)."""
     if device.type != "cuda" or nbytes <= 0 or _capturing():
         return None
-    key = (device.index, _stream_handle(stream))
+    handle = _stream_handle(stream)
+    key = (device.index, handle)
     t = _SCRATCH_CACHE.get(key)
     if t is None or t.numel() < nbytes:
-        t = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        with _on_stream(device, handle):
+            t = None                                      # the buffer it replaces goes back to this stream's pool
+            _SCRATCH_CACHE.pop(key, None)
+            t = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _SCRATCH_CACHE[key] = t
     return t
 
@@ -324,7 +366,7 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
                    work_queue=True, min_kv_len=None, static_scratch=False, stream_scratch=None,
                    probe_loads=False, single_launch=False, wavefronts=0, buffers=0, shares_per_cu=0,
                    length_feedback: Optional[LengthFeedback] = None, timeline: Optional[torch.Tensor] = None,
-                   rotate_heads=0, _planned=None) -> PreparedDecode:
+                   rotate_heads=0, fp8_fold_k_scale=False, force_balanced=False, _planned=None) -> PreparedDecode:
     """Bind all arguments of one decode call.  See ``flash_decode`` for their meaning.
 
     ``packed_out``: a ``[B, Hq, D+1]`` tensor that receives out in ``[..., :D]`` and lse (converted to its
@@ -345,8 +387,11 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     ``run_static()``, which keeps the split partials in the library's own static scratch.
     ``wavefronts`` (4 or 8) / ``buffers`` (1 or 2) are measurement aids: they override how the matrix-core split
     kernel is shaped (wavefronts per workgroup, tiles of loads under way per wavefront); ``shares_per_cu`` (1..4)
-    sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose.
+    sets how many workgroups per compute unit a balanced plan gets; 0 lets the library choose.  ``force_balanced``
+    makes the plan equal shares of the whole batch wherever the matrix-core path can run them.
     ``length_feedback``: a ``LengthFeedback`` that the call's last kernel fills (see there).
+    ``fp8_fold_k_scale=True`` (fp8 cache): the K scale multiplies the logits instead of every K value
+    (``FDK_FLAG_FP8_FOLD_K_SCALE``: faster, and off the dequantise-then-decode definition by the 16-bit rounding of K).
     ``timeline``: an int64 GPU tensor, eight values per wavefront of the split kernel; only a library built with
     ``--timeline`` writes it; ``rotate_heads`` moves the head blocks over the workgroups in that build.
     The measurement aids travel in a ``fdk_measure_args`` block (include/fdk_measure.h) that the argument block points
@@ -359,19 +404,20 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         min_kv_len)
     batch, q_heads, d = q.shape
     measure = None
-    if wavefronts or buffers or shares_per_cu or probe_loads or rotate_heads or timeline is not None:
+    if wavefronts or buffers or shares_per_cu or probe_loads or rotate_heads or force_balanced or timeline is not None:
         measure = FdkMeasureArgs()
         measure.struct_size = C.sizeof(FdkMeasureArgs)
         measure.probe_loads = 1 if probe_loads else 0
         measure.wavefronts, measure.buffers, measure.shares_per_cu = int(wavefronts), int(buffers), int(shares_per_cu)
         measure.rotate_heads = int(rotate_heads)
+        measure.force_balanced = 1 if force_balanced else 0
         if timeline is not None:
             if timeline.dtype != torch.int64 or not timeline.is_cuda or not timeline.is_contiguous():
                 raise ValueError("timeline must be a contiguous int64 GPU tensor")
             measure.timeline, measure.timeline_len = timeline.data_ptr(), timeline.numel()
         a.measure = C.addressof(measure)
-        if shares_per_cu:
-            plan = _plan_of(a)                   # this one changes the plan (workgroups, workspace)
+        if shares_per_cu or force_balanced:
+            plan = _plan_of(a)                   # these change the plan (workgroups, workspace)
     if length_feedback is not None:
         a.length_feedback = length_feedback.device_ptr
     if packed_out is not None:
@@ -411,6 +457,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         a.workspace = workspace.data_ptr()
         a.workspace_bytes = workspace.numel() * workspace.element_size()
+    if fp8_fold_k_scale:
+        a.flags |= _lib.FDK_FLAG_FP8_FOLD_K_SCALE
     if single_launch:
         a.flags |= _lib.FDK_FLAG_SINGLE_LAUNCH
     if plan.num_splits > 1 and plan.algo == "mfma" and ((work_queue and not plan.balanced) or single_launch):
@@ -426,8 +474,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
         a.counters_len = counters.numel()
     else:
         counters = None
-    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, timeline, counters,
-            measure)
+    keep = (q, k_cache, v_cache, block_table, kv_lens, k_scale, v_scale, target, lse, workspace, length_feedback, timeline, measure,
+            counters)
     return PreparedDecode(a, plan, keep, target, lse)
 
 
@@ -436,7 +484,8 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  kv_split: int = -1, max_kv_len: Optional[int] = None, k_scale: Optional[torch.Tensor] = None,
                  v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                  lse: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                 algo: str = "auto", stream=None, min_kv_len: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 algo: str = "auto", stream=None, min_kv_len: Optional[int] = None,
+                 fp8_fold_k_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Local (one GPU's share) split-KV GQA decode attention over a paged KV cache.
 
     q            [B, Hq, D] bf16/fp16, one query token per sequence
@@ -455,6 +504,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  equal shares of the tokens on the device (a single pass is as slow as its longest sequence) and
                  per-sequence chunks follow each sequence's own length; results never depend on it
     k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
+    fp8_fold_k_scale fp8 cache: apply k_scale to the logits instead of to every K value (see ``prepare_decode``)
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
     and lse = ln sum exp(scaled logits) - what the cross-rank combine consumes."""
@@ -463,7 +513,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
                           out=out, lse=lse, workspace=workspace, algo=algo, min_kv_len=min_kv_len,
-                          stream_scratch=stream if q.is_cuda else None,
+                          fp8_fold_k_scale=fp8_fold_k_scale, stream_scratch=stream if q.is_cuda else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)
 
@@ -495,6 +545,12 @@ def _drop_in_bounds(q, kv_lens, fb):
     one token per sequence; a batch that was recomposed runs its first call on the old bounds, slower but right)."""
     if fb is None or not (q.is_cuda and isinstance(kv_lens, torch.Tensor) and kv_lens.dim() == 1):
         return None, None, None
+    if _capturing():
+        # A captured call is replayed while kv_lens grows: bounds read now would be baked into the graph, and a plan
+        # that trusts them (equal chunks sized for today's length, the last one running to the end) would leave almost
+        # all tokens of a much longer replay to one workgroup per sequence.  Plan as for unknown lengths; the block
+        # is still written by every replay.
+        return fb, None, None
     lo, hi = fb.bounds(kv_lens.numel())
     return fb, lo, hi
 
