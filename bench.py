@@ -429,8 +429,8 @@ def bench_plan_sweep(args):
             best = us if best is None else min(best, us)
         return best
 
-    print("| heads | batch | kv_len | mode | library's plan | us | best alternative | us | library / best |")
-    print("|---|---|---|---|---|---|---|---|---|")
+    print("| heads | batch | kv_len | mode | library's plan | us | best alternative | us | library / best | every plan, us |")
+    print("|---|---|---|---|---|---|---|---|---|---|")
     cells = []
     for hq, hkv in heads:
         fits = [(b, n) for b in batches for n in lens_list if b * n * hkv * 2 * d * 2 <= cap_bytes]
@@ -460,14 +460,18 @@ def bench_plan_sweep(args):
                 variants += [(f"{s_} chunks", dict(kv_split=s_)) for s_ in (2, 4, 8, 16, 32) if n // s_ >= 64]
                 if b > 1:
                     variants.append(("equal shares", dict(force_balanced=True)))
-                res = []
+                prepared = []
                 for name, kw in variants:
                     rot = [tda.prepare_decode(q, k, v, t, lens, d ** -0.5, work_queue=False, **hints, **kw) for t in tables]
                     pl = rot[0].plan
                     desc = ("single pass" if pl.num_splits == 1 else
                             f"equal shares, {pl.workgroups} workgroups" if pl.balanced else
                             f"{pl.num_splits} chunks" + (" of own length" if pl.chunk_floor else "")) + f", {pl.kv_heads_per_wg} kv heads/wg"
-                    res.append((name, desc, time_call(rot)))
+                    prepared.append((name, desc, rot))
+                # two rounds over the plans, the better time of each: whichever plan runs first in a cell also pays for
+                # what is new to the cell (its table, its pages' address translations)
+                times = [min(t) for t in zip(*[[time_call(rot) for _, _, rot in prepared] for _ in range(2)])]
+                res = [(name, desc, t) for (name, desc, _), t in zip(prepared, times)]
                 lib = res[0]
                 best = min(res[1:], key=lambda r: r[2])
                 ratio = lib[2] / best[2]
@@ -476,7 +480,7 @@ def bench_plan_sweep(args):
                                   pct_of_peak=round(alg_bytes / lib[2] / 1e3 / HBM_PEAK_GBPS * 100, 1),
                                   all={r[0]: round(r[2], 2) for r in res}))
                 print(f"| {hq}/{hkv} | {b} | {n} | {mode} | {lib[1]} | {lib[2]:.1f} | {best[0]} ({best[1]}) | {best[2]:.1f} | "
-                      f"{ratio:.3f} |", flush=True)
+                      f"{ratio:.3f} | " + ", ".join(f"{r[0]} {r[2]:.1f}" for r in res[1:]) + " |", flush=True)
         del k, v
         torch.cuda.empty_cache()
     worst = sorted(cells, key=lambda c: -c["ratio"])[:12]

@@ -28,11 +28,15 @@ OBJ_DIR = PKG_DIR / "build"
 SOURCES = [
     "fdk_api.hip", "fdk_combine.hip", "fdk_splitkv_valu.hip", "fdk_splitkv_mfma.hip",
     "fdk_splitkv_valu_bf16.hip", "fdk_splitkv_valu_bf16_fp8.hip", "fdk_splitkv_valu_fp16.hip",
-    "fdk_splitkv_valu_fp16_fp8.hip", "fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip", "fdk_kv_append.hip", "fdk_probe.hip",
+    "fdk_splitkv_valu_fp16_fp8.hip", "fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip",
+    "fdk_splitkv_mfma_d64_bal.hip", "fdk_splitkv_mfma_d128_bal.hip", "fdk_splitkv_mfma_d256_bal.hip",
+    "fdk_splitkv_mfma_d64_queue.hip", "fdk_splitkv_mfma_d128_queue.hip", "fdk_splitkv_mfma_d256_queue.hip", "fdk_kv_append.hip", "fdk_probe.hip",
 ]
 
 # the translation units that contain the matrix-core split kernel: the only ones the timeline build compiles anew
-TIMELINE_SOURCES = ("fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip", "fdk_probe.hip")
+TIMELINE_SOURCES = ("fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip",
+                    "fdk_splitkv_mfma_d64_bal.hip", "fdk_splitkv_mfma_d128_bal.hip", "fdk_splitkv_mfma_d256_bal.hip",
+                    "fdk_splitkv_mfma_d64_queue.hip", "fdk_splitkv_mfma_d128_queue.hip", "fdk_splitkv_mfma_d256_queue.hip", "fdk_probe.hip")
 
 # -packed-fp32-ops off: v_pk_*_f32 forms are not to be generated for this target.
 HIPCC_FLAGS = [
@@ -75,6 +79,7 @@ def build(verbose: bool = True, jobs: int = 8, timeline: bool = False) -> Path:
             todo = [(src, obj) for src, obj in pairs if src.name in TIMELINE_SOURCES]
     if verbose:
         print(f"[fdk build] hipcc={hipcc} -> {lib_path}", flush=True)
+    todo = sorted(todo, key=lambda so: "splitkv_mfma_d" not in so[0].name)       # the longest compilations first
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as ex:
         list(ex.map(lambda so: _compile_one(hipcc, so[0], so[1], extra), todo))
     tmp = lib_path.with_suffix(".so.tmp")

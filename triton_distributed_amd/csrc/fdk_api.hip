@@ -425,6 +425,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
         return fail(FDK_ESHAPE, "grid too large (batch x splits x heads; at most 65535 sequences)");
     float* part_o = nullptr;
     float* part_lse = nullptr;
+    int2* slot_desc = nullptr;           // one per (sequence, unit), behind the partial rows
     if (!direct && a->batch > 0) {
         const size_t need = fdk_workspace_bytes(a->batch, a->num_q_heads, a->head_dim, S);
         if (!a->workspace) return fail(FDK_EWORKSPACE, "workspace is null; %zu bytes needed", need);
@@ -433,6 +434,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
             return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed for %d splits", a->workspace_bytes, need, S);
         part_o = reinterpret_cast<float*>(a->workspace);
         part_lse = part_o + rows * S * a->head_dim;
+        slot_desc = reinterpret_cast<int2*>((reinterpret_cast<uintptr_t>(part_lse + rows * S) + 7) & ~uintptr_t(7));
     }
     fdk::SplitParams& sp = r->sp;
     memset(&sp, 0, sizeof(sp));
@@ -440,7 +442,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.block_table = a->block_table; sp.kv_lens = a->kv_lens;
     sp.k_scale = a->kv_dtype == FDK_FP8_E4M3 ? a->k_scale : nullptr;
     sp.v_scale = a->kv_dtype == FDK_FP8_E4M3 ? a->v_scale : nullptr;
-    sp.part_o = part_o; sp.part_lse = part_lse;
+    sp.part_o = part_o; sp.part_lse = part_lse; sp.slot_desc = slot_desc;
     sp.out = a->out; sp.lse = a->lse;
     sp.counters = nullptr;
     sp.num_cus = num_cus;
@@ -491,7 +493,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
 
     fdk::CombineParams& cp = r->cp;
     memset(&cp, 0, sizeof(cp));
-    cp.part_o = part_o; cp.part_lse = part_lse; cp.kv_lens = a->kv_lens;
+    cp.part_o = part_o; cp.part_lse = part_lse; cp.slot_desc = slot_desc; cp.kv_lens = a->kv_lens;
     cp.out = a->out; cp.lse = a->lse;
     cp.out_sb = a->out_stride_b; cp.out_sh = a->out_stride_h; cp.lse_sb = a->lse_stride_b;
     cp.batch = a->batch; cp.hq = a->num_q_heads; cp.head_dim = a->head_dim;
@@ -579,7 +581,10 @@ size_t fdk_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t head_dim,
     if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || num_splits <= 0) return 0;
     // batch * heads * splits < 2^93 would overflow: saturate instead, so that no buffer ever passes the size check
     const unsigned __int128 rows = (unsigned __int128)batch * (unsigned __int128)num_q_heads * (unsigned __int128)num_splits;
-    const unsigned __int128 bytes = rows * ((unsigned __int128)head_dim + 1) * sizeof(float) + 255;
+    // partial rows and their lse, then (balanced plans) eight bytes per (sequence, unit) that say where a sequence's
+    // pieces are; there are at most batch x q heads units
+    const unsigned __int128 desc = (unsigned __int128)batch * (unsigned __int128)num_q_heads * 8 + 8;
+    const unsigned __int128 bytes = rows * ((unsigned __int128)head_dim + 1) * sizeof(float) + desc + 255;
     if (bytes > (unsigned __int128)SIZE_MAX) return SIZE_MAX;
     return (size_t)bytes & ~(size_t)255;
 }

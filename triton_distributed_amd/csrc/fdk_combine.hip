@@ -8,6 +8,8 @@
 // per split loads its lse, the wavefront reduces max and sum with cross-lane ops, and the weighted
 // accumulation over the partial rows then runs with independent loads.  One wavefront per
 // (sequence, q head); each lane owns head_dim/64 adjacent output columns.
+//   combine_slots_kernel  the same merge for balanced plans (equal shares of the whole batch), whose pieces are whole
+//                         slots of adjacent rows: one workgroup per (sequence, unit) with 16-byte loads
 #include "fdk_device.h"
 
 namespace fdk {
@@ -48,55 +50,18 @@ struct PartRows {
     int live;
 };
 
+// chunk mode: split c holds tokens [c*chunk, ...) - the split kernel wrote exactly the live ones
 template <int D>
 __device__ __forceinline__ PartRows locate_rows(const CombineParams& p, int b, int h) {
     PartRows r;
-    if (!p.balanced) {
-        // chunk mode: split c holds tokens [c*chunk, ...) - the split kernel wrote exactly the live ones
-        const int kv_len = min(p.kv_lens[b], p.max_tokens);
-        const int64_t row = (int64_t)b * p.hq + h;
-        const int chunk = chunk_tokens_of(kv_len, p.num_splits, p.chunk, p.chunk_floor);
-        r.live = min(p.num_splits, (kv_len + chunk - 1) / chunk);
-        r.o = p.part_o + row * p.num_splits * D;
-        r.lse = p.part_lse + row * p.num_splits;
-        r.o_step = D;
-        r.lse_step = 1;
-        return r;
-    }
-    // balanced mode: redo the split kernel's partition.  The sequences, in granules laid end to end, are cut
-    // into `shares` equal parts (the first `rem` one granule longer); sequence b spans granules
-    // [before, before + mine); the piece of share wc for unit u is in slot (wc + b) * units + u.
-    const int lane = threadIdx.x & 63;
-    const int units = p.hg_blocks * p.head_tiles;
-    // (a sequence with tokens counts for p.piece_cost granules more, in front of its own: see the split kernel)
-    int total = 0, before = 0;
-    for (int b0 = 0; b0 < p.batch; b0 += 64) {
-        const int bb = b0 + lane;
-        int g = bb < p.batch ? (max(min(p.kv_lens[bb], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule : 0;
-        if (g > 0) g += p.piece_cost;
-        total += g;
-        before += bb < b ? g : 0;
-    }
-    total = wave_sum_i32(total);
-    before = wave_sum_i32(before) + p.piece_cost;          // where the granules of sequence b begin
-    const int mine = (max(min(p.kv_lens[b], p.max_tokens), 0) + kBalanceGranule - 1) / kBalanceGranule;
-    const int kvh = h / p.group, hin = h % p.group;
-    const int u = (kvh / p.kv_heads_per_wg) * p.head_tiles + hin / 16;
-    const int row_in_slot = (kvh % p.kv_heads_per_wg) * p.heads_per_tile + hin % 16;
-    r.o_step = (int64_t)units * p.rows_per_slot * D;
-    r.lse_step = units * p.rows_per_slot;
-    r.live = 0;
-    r.o = p.part_o;
-    r.lse = p.part_lse;
-    if (mine == 0) return r;
-    const int shares = min(p.workgroups / units, total);
-    const int q = total / shares, rem = total % shares;
-    auto share_of = [&](int x) { return x < rem * (q + 1) ? x / (q + 1) : rem + (x - rem * (q + 1)) / q; };
-    const int wc_first = share_of(before), wc_last = share_of(before + mine - 1);
-    const int64_t row0 = ((int64_t)(wc_first + b) * units + u) * p.rows_per_slot + row_in_slot;
-    r.live = wc_last - wc_first + 1;
-    r.o = p.part_o + row0 * D;
-    r.lse = p.part_lse + row0;
+    const int kv_len = min(p.kv_lens[b], p.max_tokens);
+    const int64_t row = (int64_t)b * p.hq + h;
+    const int chunk = chunk_tokens_of(kv_len, p.num_splits, p.chunk, p.chunk_floor);
+    r.live = min(p.num_splits, (kv_len + chunk - 1) / chunk);
+    r.o = p.part_o + row * p.num_splits * D;
+    r.lse = p.part_lse + row * p.num_splits;
+    r.o_step = D;
+    r.lse_step = 1;
     return r;
 }
 
@@ -113,8 +78,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     // are never used) - the kernel is a chain of dependent memory round trips, this removes one or two.
     constexpr int kPre = 8;
     float pre[kPre][EPL];
-    float lse_early = 0.f;                       // chunk mode: lse of split `lane`, requested just as early
-    if (!p.balanced) {
+    float lse_early = 0.f;                       // lse of split `lane`, requested just as early
+    {
         const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
 #pragma unroll
         for (int j = 0; j < kPre; ++j)
@@ -125,11 +90,6 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     const int live = pr.live;
     const float* lse_row = pr.lse;
     const float* o_row = pr.o + EPL * lane;
-    if (p.balanced) {
-#pragma unroll
-        for (int j = 0; j < kPre; ++j)
-            if (j < live) Vec<EPL>::load(o_row + j * pr.o_step, pre[j]);
-    }
 
     float m_run = -INFINITY, l_run = 0.f;
     float acc[EPL];
@@ -137,7 +97,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const CombineParams p) {
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
     for (int s0 = 0; s0 < live; s0 += 64) {
         const int n = min(64, live - s0);
-        const float my = lane < n ? (!p.balanced && s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step]) * kLog2e
+        const float my = lane < n ? (s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step]) * kLog2e
                                   : -INFINITY;   // log2 units
         const float m_blk = wave_max(my);
         const float m_new = fmaxf(m_run, m_blk);
@@ -201,7 +161,7 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     constexpr int kPre = 16;
     float pre[kPre][EPL];
     float lse_early = 0.f;
-    if (!p.balanced) {
+    {
         const float* o_early = p.part_o + row * p.num_splits * D + EPL * lane;
 #pragma unroll
         for (int j = 0; j < kPre; ++j)
@@ -212,16 +172,11 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     const int live = pr.live;
     const float* lse_row = pr.lse;
     const float* o_row = pr.o + EPL * lane;
-    if (p.balanced) {
-#pragma unroll
-        for (int j = 0; j < kPre; ++j)
-            if (wave + kRowsPerWg * j < live) Vec<EPL>::load(o_row + (wave + kRowsPerWg * j) * pr.o_step, pre[j]);
-    }
 
     float m = -INFINITY;
     float my_first = -INFINITY;                    // lse of split `lane`, kept for the second pass
     for (int s0 = 0; s0 < live; s0 += 64) {
-        const float my = s0 + lane < live ? (!p.balanced && s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step])
+        const float my = s0 + lane < live ? (s0 == 0 ? lse_early : lse_row[(s0 + lane) * pr.lse_step])
                                           : -INFINITY;
         if (s0 == 0) my_first = my;
         m = fmaxf(m, wave_max(my));
@@ -278,6 +233,74 @@ __global__ __launch_bounds__(256) void combine_wide_kernel(const CombineParams p
     }
     if (p.length_feedback && row == 0)
         store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
+}
+
+// Balanced plans.  The pieces of a (sequence, unit) are whole slots - rows_per_slot adjacent partial rows, one per
+// (kv head of the block, q head of the tile) - in consecutive shares, and the split kernel has left {first share,
+// live pieces} for every (sequence, unit) that holds tokens.  One workgroup per (sequence, unit); a thread owns four
+// adjacent columns of one row, requests that row's lse values and its 16 bytes of up to eight pieces at once, and
+// merges them by itself: no cross-lane traffic, no pass over kv_lens, one dependent round trip after the descriptor.
+template <int D>
+__global__ __launch_bounds__(1024) void combine_slots_kernel(const CombineParams p) {
+    constexpr int LPR = D / 4;                    // threads per row
+    constexpr int NB = 8;                         // pieces per batch of loads
+    const int units = p.hg_blocks * p.head_tiles;
+    const int b = blockIdx.x / units, u = blockIdx.x % units;
+    const int2 desc = p.slot_desc[blockIdx.x];                  // (garbage for a sequence without tokens: not used)
+    const int kv_len = p.kv_lens[b];
+    const int hgb = u / p.head_tiles, ht = u % p.head_tiles;
+    const int heads_here = min(16, p.group - ht * 16);
+    const int c4 = threadIdx.x % LPR;
+    const int64_t piece_step = (int64_t)units * p.rows_per_slot;                 // rows from one piece to the next
+    for (int r = threadIdx.x / LPR; r < p.rows_per_slot; r += p.rows_per_pass) {
+        const int hl = r / p.heads_per_tile, g = r % p.heads_per_tile;
+        if (g >= heads_here) continue;                                       // the last tile of a group may be short
+        const int hq = (hgb * p.kv_heads_per_wg + hl) * p.group + ht * 16 + g;
+        const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float inv = 0.f, lse = -INFINITY;                                    // no tokens: out = 0, lse = -inf
+        if (kv_len > 0) {
+            const int64_t row0 = ((int64_t)(desc.x + b) * units + u) * p.rows_per_slot + r;
+            const float* lse_p = p.part_lse + row0;
+            const float* o_p = p.part_o + row0 * D + 4 * c4;
+            float m_run = -INFINITY, l_run = 0.f;
+            for (int s0 = 0; s0 < desc.y; s0 += NB) {
+                float ls[NB];
+                float4 o[NB];
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    ls[j] = -INFINITY;
+                    o[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (s0 + j < desc.y) {
+                        ls[j] = lse_p[(s0 + j) * piece_step];
+                        o[j] = *reinterpret_cast<const float4*>(o_p + (s0 + j) * piece_step * D);
+                    }
+                }
+                float m_new = m_run;
+#pragma unroll
+                for (int j = 0; j < NB; ++j) m_new = fmaxf(m_new, ls[j] * kLog2e);     // finite: a live piece holds a token
+                const float alpha = fast_exp2(m_run - m_new);
+                l_run *= alpha;
+                acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const float w = fast_exp2(ls[j] * kLog2e - m_new);                  // 0 past the last piece
+                    l_run += w;
+                    acc.x += w * o[j].x; acc.y += w * o[j].y; acc.z += w * o[j].z; acc.w += w * o[j].w;
+                }
+                m_run = m_new;
+            }
+            inv = 1.0f / l_run;
+            lse = (m_run + fast_log2(l_run)) * kLn2;
+        }
+        store_out4(p.out, ob + 4 * c4, make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv), p.out_dtype);
+        if (c4 == 0) {
+            if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse;
+            if (p.pack_lse) store_out(p.out, ob + D, lse, p.out_dtype);
+        }
+    }
+    if (p.length_feedback && blockIdx.x == 0 && threadIdx.x < 64)
+        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, threadIdx.x);
 }
 
 __device__ __forceinline__ float load_any(const void* base, int64_t idx, int dtype) {
@@ -345,9 +368,22 @@ __global__ __launch_bounds__(256) void combine_ranks_kernel(const CombineRanksPa
 int launch_combine(const CombineParams& p, hipStream_t stream) {
     const int64_t rows = (int64_t)p.batch * p.hq;
     if (rows == 0) return 0;
-    // pieces of a row: the split count, or in balanced mode about shares / sequences
-    const int units = p.hg_blocks * p.head_tiles;
-    const bool wide = (p.balanced ? p.workgroups / (units > 0 ? units : 1) / (p.batch > 0 ? p.batch : 1) + 1 : p.num_splits) > 8;
+    if (p.balanced) {
+        const int units = p.hg_blocks * p.head_tiles;
+        const dim3 grid((unsigned)(p.batch * units));
+        const int lpr = p.head_dim / 4;
+        const dim3 block((unsigned)(p.rows_per_slot * lpr > 1024 ? 1024 : p.rows_per_slot * lpr < 64 ? 64 : p.rows_per_slot * lpr));
+        CombineParams q = p;
+        q.rows_per_pass = (int32_t)block.x / lpr;
+        switch (p.head_dim) {
+            case 64: hipLaunchKernelGGL(combine_slots_kernel<64>, grid, block, 0, stream, q); break;
+            case 128: hipLaunchKernelGGL(combine_slots_kernel<128>, grid, block, 0, stream, q); break;
+            case 256: hipLaunchKernelGGL(combine_slots_kernel<256>, grid, block, 0, stream, q); break;
+            default: return (int)hipErrorInvalidValue;
+        }
+        return (int)hipGetLastError();
+    }
+    const bool wide = p.num_splits > 8;
     const dim3 grid((unsigned)(wide ? rows : (rows + kRowsPerWg - 1) / kRowsPerWg));
 #define FDK_COMBINE_LAUNCH(DV)                                                                     \
     do {                                                                                           \

@@ -28,6 +28,8 @@ struct SplitParams {
     void* out;        // final output, written directly when S == 1
     float* lse;       // may be null
     int32_t* counters;  // zeroed scratch counters of the work queue: [0] head, [1] finished workgroups
+    int2* slot_desc;    // balanced mode: where the pieces of (sequence, unit) are - {first share, live pieces} - written
+                        // by the piece that holds the sequence's first token, read by the combine
     int64_t q_sb, q_sh;
     int64_t k_sp, k_st, k_sh;  // page / token / head strides, elements
     int64_t v_sp, v_st, v_sh;
@@ -45,6 +47,12 @@ struct SplitParams {
     int32_t direct;                 // 1: single split, write the final (out, lse) instead of partials
     int32_t persistent, total_items, num_cus;
     int32_t balanced, workgroups;   // balanced mode: the KV ranges are cut into `workgroups` equal shares
+    // What the launch was given, as arguments: the kernels must not read gridDim / blockDim where a result is on the way
+    // to the first loads - those live in the hidden arguments, which are fetched only when first used, and a fetch from
+    // the argument buffer that is not part of the batch at kernel entry costs a round trip of its own (measured 1.4 us).
+    int32_t shares;                 // balanced mode: gridDim.y
+    int32_t grid_x;                 // gridDim.x
+    int32_t wavefronts;             // blockDim.x / 64
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
@@ -66,6 +74,7 @@ struct SplitParams {
 struct CombineParams {
     const float* part_o;
     const float* part_lse;
+    const int2* slot_desc;          // balanced mode: as in SplitParams
     const int32_t* kv_lens;
     void* out;
     float* lse;
@@ -79,6 +88,7 @@ struct CombineParams {
     // balanced mode (see the split kernel): where the pieces of a (sequence, head) row are
     int32_t balanced, workgroups;
     int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile, piece_cost;
+    int32_t rows_per_pass;          // balanced mode: rows of a slot the workgroup covers at once (blockDim.x / (head_dim / 4))
     int32_t* length_feedback;       // as in SplitParams (null: nothing is stored)
     int32_t feedback_epoch;
 };

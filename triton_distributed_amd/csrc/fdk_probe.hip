@@ -49,8 +49,15 @@ __global__ __launch_bounds__(256) void linear_read_kernel(const u32x4_t* __restr
 int launch_splitkv_mfma_probe(const SplitParams& p, int kv_dtype, hipStream_t stream) {
     if (p.head_dim != 128) return (int)hipErrorInvalidValue;
     // the q dtype does not matter to the loads: fp16 rows have the same bytes as bf16 rows
-    return kv_dtype == FDK_FP8_E4M3 ? launch_pm<FDK_BF16, true, 128, true>(p, stream)
-                                    : launch_pm<FDK_BF16, false, 128, true>(p, stream);
+    const bool fp8 = kv_dtype == FDK_FP8_E4M3;
+    switch (mfma_work_mode(p)) {
+        case WM_SHARES:
+            return fp8 ? launch_pm<FDK_BF16, true, 128, true, WM_SHARES>(p, stream) : launch_pm<FDK_BF16, false, 128, true, WM_SHARES>(p, stream);
+        case WM_QUEUE:
+            return fp8 ? launch_pm<FDK_BF16, true, 128, true, WM_QUEUE>(p, stream) : launch_pm<FDK_BF16, false, 128, true, WM_QUEUE>(p, stream);
+        default:
+            return fp8 ? launch_pm<FDK_BF16, true, 128, true, WM_ONE>(p, stream) : launch_pm<FDK_BF16, false, 128, true, WM_ONE>(p, stream);
+    }
 }
 
 int launch_linear_read(const void* buf, size_t bytes, int nontemporal, int workgroups, uint32_t* sink, hipStream_t stream) {

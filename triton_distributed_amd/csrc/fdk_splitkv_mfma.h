@@ -228,8 +228,13 @@ __device__ __forceinline__ void merge_rows(const SplitParams& p, const int64_t (
 
 // PROBE: the load pipeline alone - the same pieces, addresses and load instructions in the same order, but what
 // arrives is only folded into a checksum: how fast the memory system serves this call's access pattern.
-template <int QDT, bool FP8, int PM, int NBUF, int D, bool PROBE = false>
+// MODE: how pieces are handed out - a kernel for each, see "work distribution" below.
+enum WorkMode { WM_ONE = 0,     // one piece per workgroup: single pass, per-sequence chunks
+                WM_QUEUE = 1,   // chunk mode, a fixed set of workgroups pulls the pieces from a queue
+                WM_SHARES = 2 };// balanced mode: equal shares of the whole batch
+template <int QDT, bool FP8, int PM, int NBUF, int D, bool PROBE = false, int MODE = WM_ONE>
 __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) {
+    constexpr bool BAL = MODE == WM_SHARES;
     using M = Mma<QDT>;
     using P2 = Pack2<QDT>;
     using R = Regs<FP8, D>;
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     const int lrow = lane / LPR;               // row of this lane within a load
     const int lpiece = lane % LPR;             // 16-byte piece of the row
 
-    const int nw = blockDim.x >> 6;
+    const int nw = p.wavefronts;               // (= blockDim.x / 64; see SplitParams)
     const int nh = p.hg_per_wg;                // kv heads per workgroup
     const int ti_n = nw / nh;                  // wavefronts interleaving the tiles of one kv head
     const int hl = wave % nh;
@@ -346,7 +351,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
         return;
     }
     const int c_end = min(c_limit, kv_len);
-    if (!p.balanced && p.fused) {                                                       // chunks that hold tokens
+    if (!BAL && p.fused) {                                                              // chunks that hold tokens
         const int chunk = chunk_tokens_of(kv_len, p.num_splits, p.chunk, p.chunk_floor);
         mr.live = min(p.num_splits, (kv_len + chunk - 1) / chunk);
     }
@@ -760,63 +765,180 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     // counters[1] counts finished workgroups, and the last one to finish puts both back to zero.  The first item
     // of every workgroup is its own index.
     // Balanced mode: the sequences, counted in granules of kGranule tokens and laid end to end, are cut into
-    // gridDim.y equal shares (fewer if there are fewer granules), units = (kv-head block, q-head tile)
+    // p.shares (= gridDim.y) equal shares (fewer if there are fewer granules), units = (kv-head block, q-head tile)
     // pairs of a sequence; workgroup (share wc, unit u) = (blockIdx.y, blockIdx.x) works its share off for its unit, sequence
     // by sequence.  Its partial rows for sequence b go to slot (wc + b) * units + u: pieces are ordered by
     // (wc, b) with at least one of the two growing from one piece to the next, so the slot is unique, and the
     // pieces of a sequence occupy consecutive wc.  Neighbouring workgroups read the same tokens of neighbouring
     // heads.  Every wavefront derives the same partition from kv_lens.
-    if (!p.balanced && !p.persistent) {
-        // The common chunk-mode case is kept free of the loop below: straight-line code lets the compiler
-        // overlap the first loads of the piece (about a microsecond per workgroup on MI355X).
-        // grid = (head blocks x head tiles, splits, sequences): the piece follows from the block index without a
-        // division, so the table and q loads of the piece can be requested as soon as the arguments are there.
-        // (Workgroups are handed out in x-major order: neighbours still read neighbouring heads of the same tokens.)
-        const int split = blockIdx.y, pb = blockIdx.z;
-        int ht = 0, hgb = blockIdx.x;
+    //
+    // The modes are kernels of their own (template parameter MODE): the code of one does not get in the way of the
+    // others' registers and schedule.  In all of them the FIRST piece of a workgroup - in chunk mode without a queue
+    // its only one - runs through straight-line code: that lets the compiler put the piece's first loads ahead of everything that
+    // does not feed them.  A loop for the pieces after it is entered only by workgroups that have more (a share that
+    // holds the end of one sequence and the beginning of the next; the work queue): what the compiler computes once in
+    // front of a loop - several hundred instructions here - would otherwise stand between every workgroup and its
+    // first loads (measured in balanced mode: first loads 2.7 us after the start of the kernel instead of 1.9 us).
+    if constexpr (MODE == WM_ONE) {
+        {
+            // grid = (head blocks x head tiles, splits, sequences): the piece follows from the block index without a
+            // division, so the table and q loads of the piece can be requested as soon as the arguments are there.
+            // (Workgroups are handed out in x-major order: neighbours still read neighbouring heads of the same tokens.)
+            const int split = blockIdx.y, pb = blockIdx.z;
+            int ht = 0, hgb = blockIdx.x;
 #ifdef FDK_TIMELINE
-        if (p.head_tiles == 1) hgb = (int)((blockIdx.x + (unsigned)p.timeline_rotate) % gridDim.x);
+            if (p.head_tiles == 1) hgb = (int)((blockIdx.x + (unsigned)p.timeline_rotate) % (unsigned)p.grid_x);
 #endif
-        if (p.head_tiles > 1) {
-            ht = blockIdx.x % p.head_tiles;
-            hgb = blockIdx.x / p.head_tiles;
+            if (p.head_tiles > 1) {
+                ht = blockIdx.x % p.head_tiles;
+                hgb = blockIdx.x / p.head_tiles;
+            }
+            // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
+            const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
+            // (chunks that follow the sequence's own length: the first table read then waits for kv_lens, one more
+            // round trip before the first rows - the price of not needing a length bound from the host)
+            int chunk = p.chunk;
+            if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
+            run_piece(pb, hgb, ht, split * chunk, split == p.num_splits - 1 ? p.max_tokens : split * chunk + chunk,
+                      unit_row0 + (int64_t)hl * p.group * p.num_splits + split, p.num_splits,
+                      MergeRows{unit_row0, 1, (int64_t)p.group * p.num_splits, p.num_splits, 0});
+            if (p.length_feedback && (blockIdx.x | blockIdx.y | blockIdx.z) == 0 && wave == 0)
+                store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
+            return;
         }
-        // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
-        const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
-        // (chunks that follow the sequence's own length: the first table read then waits for kv_lens, one more
-        // round trip before the first rows - the price of not needing a length bound from the host)
-        int chunk = p.chunk;
-        if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
-        run_piece(pb, hgb, ht, split * chunk, split == p.num_splits - 1 ? p.max_tokens : split * chunk + chunk,
-                  unit_row0 + (int64_t)hl * p.group * p.num_splits + split, p.num_splits,
-                  MergeRows{unit_row0, 1, (int64_t)p.group * p.num_splits, p.num_splits, 0});
-        if (p.length_feedback && (blockIdx.x | blockIdx.y | blockIdx.z) == 0 && wave == 0)
+    } else if constexpr (MODE == WM_QUEUE) {
+        // work queue (single-launch form with a forced split count: it ends the call, so it reports the lengths)
+        if (p.length_feedback && blockIdx.x == 0 && wave == 0)
             store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
-        return;
-    }
-    // length feedback where this kernel is the last of the call (the single-launch form: no combine follows)
-    if (p.length_feedback && (blockIdx.x | blockIdx.y | blockIdx.z) == 0 && wave == 0)
-        store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
-    const int units = p.hg_blocks * p.head_tiles;
-    // A sequence counts for its granules plus p.piece_cost more in front of them (none if it is empty): every
-    // sequence a share begins costs its workgroup a fixed time (table and q loads before the first rows, the merge
-    // of the wavefronts after the last), and a share that starts several sequences gets fewer tokens for it.
-    const int pc = p.piece_cost;
-    auto granules_of = [&](int bb) {
-        const int g = (max(min(as_const(p.kv_lens)[bb], p.max_tokens), 0) + kGranule - 1) / kGranule;
-        return g > 0 ? g + pc : 0;
-    };
-    int item = blockIdx.x;                        // chunk mode: current item
-    int x = 0, hi = 0;                            // balanced mode: next granule, end of this workgroup's share
-    int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
-    const int wc = blockIdx.y, bu = blockIdx.x;   // balanced mode: grid = (units, shares); queue: grid = (workgroups)
-    int share_q = 1, share_r = 0;                 // balanced mode: granules per share, shares with one more
-    if (p.balanced) {
+        int item = blockIdx.x;
+        if (item >= p.total_items) return;
+        for (;;) {
+            int wg = item;
+            int ht = wg % p.head_tiles;
+            wg /= p.head_tiles;
+            int hgb = wg % p.hg_blocks;
+            wg /= p.hg_blocks;
+            const int split = wg % p.num_splits;
+            int pb = wg / p.num_splits;
+            int chunk = p.chunk;
+            if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
+            int c_start = split * chunk;
+            int c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + chunk;
+            int64_t prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
+            MergeRows mr;
+            mr.live = 0;                                              // from kv_len, inside run_piece
+            mr.base = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
+            mr.piece_step = 1;
+            mr.hl_step = (int64_t)p.group * p.num_splits;
+            mr.g_step = p.num_splits;
+            // everything that describes the piece is wave-uniform: keep it in scalar registers
+            pb = __builtin_amdgcn_readfirstlane(pb);
+            hgb = __builtin_amdgcn_readfirstlane(hgb);
+            ht = __builtin_amdgcn_readfirstlane(ht);
+            c_start = __builtin_amdgcn_readfirstlane(c_start);
+            c_limit = __builtin_amdgcn_readfirstlane(c_limit);
+            prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(prow0 >> 32)) << 32) |
+                    (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)prow0);
+            run_piece(pb, hgb, ht, c_start, c_limit, prow0, p.num_splits, mr);
+            __syncthreads();                                          // the LDS scratch is reused by the next piece
+            if (threadIdx.x == 0) s_next[0] = p.grid_x + atomicAdd(p.counters, 1);
+            __syncthreads();
+            item = s_next[0];
+            // unsigned: a queue head that was not zero on entry ends the queue instead of yielding a negative item
+            if ((unsigned)item >= (unsigned)p.total_items) break;
+        }
+        if (threadIdx.x == 0) {                       // leave the counters at zero
+            const int done = atomicAdd(p.counters + 1, 1);
+            if (done == p.grid_x - 1) {
+                atomicExch(p.counters, 0);
+                atomicExch(p.counters + 1, 0);
+            }
+        }
+    } else {
+        struct Piece {
+            int pb, hgb, ht, c_start, c_limit;
+            int64_t prow0;
+            MergeRows mr;
+        };
+        const int units = p.hg_blocks * p.head_tiles;
+        // A sequence counts for its granules plus p.piece_cost more in front of them (none if it is empty): every
+        // sequence a share begins costs its workgroup a fixed time (table and q loads before the first rows, the merge
+        // of the wavefronts after the last), and a share that starts several sequences gets fewer tokens for it.
+        const int pc = p.piece_cost;
+        auto granules_of = [&](int bb) {
+            const int g = (max(min(as_const(p.kv_lens)[bb], p.max_tokens), 0) + kGranule - 1) / kGranule;
+            return g > 0 ? g + pc : 0;
+        };
+        int x = 0, hi = 0;                            // next granule, end of this workgroup's share
+        int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
+        const int wc = blockIdx.y, bu = blockIdx.x;   // grid = (units, shares)
+        int share_q = 1, share_r = 0;                 // granules per share, shares with one more
+        // the piece of sequence b in this workgroup's share, and where the share's part of the sequence ends
+        auto piece_of = [&](int& piece_end) {
+            Piece pp;
+            piece_end = min(before + gb, hi);
+            pp.pb = b;
+            pp.hgb = bu;
+            pp.ht = 0;
+            if (p.head_tiles > 1) {
+                pp.hgb = bu / p.head_tiles;
+                pp.ht = bu % p.head_tiles;
+            }
+            pp.c_start = max(x - before - pc, 0) * kGranule;                // the first pc positions hold no tokens
+            pp.c_limit = (piece_end - before - pc) * kGranule;              // <= 0: nothing of this sequence in the share
+            const int64_t slot = (int64_t)(wc + b) * units + bu;
+            pp.prow0 = slot * p.rows_per_slot + hl * p.heads_per_tile;
+            // the shares that hold granules [before, before + gb) of this sequence (the first share_r shares
+            // have share_q + 1 granules)
+            auto share_of = [&](int g) {
+                const int big = share_r * (share_q + 1);
+                return g < big ? g / (share_q + 1) : share_r + (g - big) / share_q;
+            };
+            pp.mr = MergeRows{0, 0, 0, 0, 0};
+            if (p.fused) {                       // (two integer divisions each: not on the way to the first loads)
+                const int wc_first = share_of(before + pc);
+                pp.mr.live = share_of(before + gb - 1) - wc_first + 1;
+                pp.mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
+                pp.mr.piece_step = (int64_t)units * p.rows_per_slot;
+                pp.mr.hl_step = p.heads_per_tile;
+                pp.mr.g_step = 1;
+            }
+            // everything that describes the piece is wave-uniform: keep it in scalar registers
+            pp.pb = __builtin_amdgcn_readfirstlane(pp.pb);
+            pp.hgb = __builtin_amdgcn_readfirstlane(pp.hgb);
+            pp.ht = __builtin_amdgcn_readfirstlane(pp.ht);
+            pp.c_start = __builtin_amdgcn_readfirstlane(pp.c_start);
+            pp.c_limit = __builtin_amdgcn_readfirstlane(pp.c_limit);
+            pp.prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(pp.prow0 >> 32)) << 32) |
+                       (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)pp.prow0);
+            return pp;
+        };
+        // After a piece: the piece that holds the first token of its sequence says where the combine finds the
+        // sequence's pieces for this unit - its own share and the number of shares up to the one with the last token
+        // (after the piece, so that the divisions are not on the way to its loads); then on to the next sequence that
+        // has tokens.  False: the share is worked off.
+        auto next_piece = [&](const Piece& pp, int piece_end) {
+            if (!p.fused && pp.c_start == 0 && pp.c_limit > 0 && threadIdx.x == 0) {
+                const int big = share_r * (share_q + 1);
+                const int g_last = before + gb - 1;
+                const int wc_last = g_last < big ? g_last / (share_q + 1) : share_r + (g_last - big) / share_q;
+                p.slot_desc[b * units + bu] = make_int2(wc, wc_last - wc + 1);
+            }
+            x = piece_end;
+            if (x >= hi) return false;
+            before += gb;
+            do {                                                          // one exists: granule x < hi is somewhere
+                b = min(b + 1, p.batch - 1);
+                gb = granules_of(b);
+            } while (gb == 0 && b + 1 < p.batch);
+            return gb != 0;
+        };
+        // every wavefront derives the partition: a prefix sum over the sequences' granules, 64 at a time
         const int g_first = lane < p.batch ? granules_of(lane) : 0;          // sequences 0..63
         const int incl_first = wave_scan_i32(g_first);
         int total = __builtin_amdgcn_readlane(incl_first, 63);
         for (int b0 = 64; b0 < p.batch; b0 += 64) total += wave_sum_i32(b0 + lane < p.batch ? granules_of(b0 + lane) : 0);
-        const int shares = min((int)gridDim.y, total);
+        const int shares = min(p.shares, total);
         if (p.fused && wc == 0 && tix == 0) {
             // no piece, hence no merge, ever touches a sequence without tokens: the first share writes those rows
             for (int b0 = 0; b0 < p.batch; b0 += 64) {
@@ -829,6 +951,8 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
                 }
             }
         }
+        if (p.length_feedback && (bu | wc) == 0 && wave == 0)          // single-launch form: no combine follows
+            store_length_bounds(p.length_feedback, p.kv_lens, p.batch, p.max_tokens, p.feedback_epoch, lane);
         if (wc >= shares) return;                                            // also total == 0
         const int q = total / shares, r = total % shares;
         share_q = q;
@@ -849,104 +973,34 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
             }
             run += __builtin_amdgcn_readlane(incl, 63);
         }
-    } else if (item >= p.total_items) {
-        return;
-    }
-    for (;;) {
-        int pb, hgb, ht, c_start, c_limit, prow_step;
-        int64_t prow0;
         int piece_end = 0;
-        MergeRows mr;
-        if (p.balanced) {
-            piece_end = min(before + gb, hi);
-            pb = b;
-            hgb = bu;
-            ht = 0;
-            if (p.head_tiles > 1) {
-                hgb = bu / p.head_tiles;
-                ht = bu % p.head_tiles;
-            }
-            c_start = max(x - before - pc, 0) * kGranule;                // the first pc positions hold no tokens
-            c_limit = (piece_end - before - pc) * kGranule;              // <= 0: nothing of this sequence in the share
-            const int64_t slot = (int64_t)(wc + b) * units + bu;
-            prow0 = slot * p.rows_per_slot + hl * p.heads_per_tile;
-            prow_step = 1;
-            // the shares that hold granules [before, before + gb) of this sequence (the first share_r shares
-            // have share_q + 1 granules)
-            auto share_of = [&](int g) {
-                const int big = share_r * (share_q + 1);
-                return g < big ? g / (share_q + 1) : share_r + (g - big) / share_q;
-            };
-            mr = MergeRows{0, 0, 0, 0, 0};
-            if (p.fused) {                       // (two integer divisions each: not on the way to the first loads)
-                const int wc_first = share_of(before + pc);
-                mr.live = share_of(before + gb - 1) - wc_first + 1;
-                mr.base = ((int64_t)(wc_first + b) * units + bu) * p.rows_per_slot;
-                mr.piece_step = (int64_t)units * p.rows_per_slot;
-                mr.hl_step = p.heads_per_tile;
-                mr.g_step = 1;
-            }
-        } else {
-            int wg = item;
-            ht = wg % p.head_tiles;
-            wg /= p.head_tiles;
-            hgb = wg % p.hg_blocks;
-            wg /= p.hg_blocks;
-            const int split = wg % p.num_splits;
-            pb = wg / p.num_splits;
-            int chunk = p.chunk;
-            if (p.chunk_floor) chunk = chunk_tokens_of(min(as_const(p.kv_lens)[pb], p.max_tokens), p.num_splits, p.chunk, p.chunk_floor);
-            c_start = split * chunk;
-            c_limit = split == p.num_splits - 1 ? p.max_tokens : c_start + chunk;
-            prow0 = ((int64_t)pb * p.hq + (hgb * nh + hl) * p.group + ht * 16) * p.num_splits + split;
-            prow_step = p.num_splits;
-            mr.live = 0;                                              // from kv_len, inside run_piece
-            mr.base = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
-            mr.piece_step = 1;
-            mr.hl_step = (int64_t)p.group * p.num_splits;
-            mr.g_step = p.num_splits;
-        }
-        // everything that describes the piece is wave-uniform: keep it in scalar registers
-        pb = __builtin_amdgcn_readfirstlane(pb);
-        hgb = __builtin_amdgcn_readfirstlane(hgb);
-        ht = __builtin_amdgcn_readfirstlane(ht);
-        c_start = __builtin_amdgcn_readfirstlane(c_start);
-        c_limit = __builtin_amdgcn_readfirstlane(c_limit);
-        prow_step = __builtin_amdgcn_readfirstlane(prow_step);
-        prow0 = ((int64_t)__builtin_amdgcn_readfirstlane((int)(prow0 >> 32)) << 32) |
-                (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)prow0);
-        if (!p.balanced || c_limit > 0) run_piece(pb, hgb, ht, c_start, c_limit, prow0, prow_step, mr);
-        if (p.balanced) {
-            x = piece_end;
-            if (x >= hi) return;
-            before += gb;                                             // on to the next sequence that has tokens
-            do {                                                      // one exists: granule x < hi is somewhere
-                b = min(b + 1, p.batch - 1);
-                gb = granules_of(b);
-            } while (gb == 0 && b + 1 < p.batch);
-            if (gb == 0) return;
+        const Piece first = piece_of(piece_end);
+        if (first.c_limit > 0) run_piece(first.pb, first.hgb, first.ht, first.c_start, first.c_limit, first.prow0, 1, first.mr);
+        if (!next_piece(first, piece_end)) return;
+        for (;;) {
             __syncthreads();                                          // the LDS scratch is reused by the next piece
-        } else {
-            if (!p.persistent) return;
-            __syncthreads();
-            if (threadIdx.x == 0) s_next[0] = (int)gridDim.x + atomicAdd(p.counters, 1);
-            __syncthreads();
-            item = s_next[0];
-            // unsigned: a queue head that was not zero on entry ends the queue instead of yielding a negative item
-            if ((unsigned)item >= (unsigned)p.total_items) break;
-        }
-    }
-    if (threadIdx.x == 0) {                       // persistent chunk mode: leave the counters at zero
-        const int done = atomicAdd(p.counters + 1, 1);
-        if (done == (int)gridDim.x - 1) {
-            atomicExch(p.counters, 0);
-            atomicExch(p.counters + 1, 0);
+            const Piece pp = piece_of(piece_end);
+            if (pp.c_limit > 0) run_piece(pp.pb, pp.hgb, pp.ht, pp.c_start, pp.c_limit, pp.prow0, 1, pp.mr);
+            if (!next_piece(pp, piece_end)) return;
         }
     }
 }
 
-template <int QDT, bool FP8, int D, bool PROBE = false>
+// Whether the call runs as a work queue: whenever the KV range is split into per-sequence chunks, the caller provided
+// counters and there are more pieces than are resident at once - pieces of a ragged batch differ in length, and a
+// queue keeps every compute unit busy until the end.
+inline bool mfma_runs_as_queue(const SplitParams& p) {
+    const int hg_per_wg = (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) ? 1 : p.hg_per_wg;
+    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + 15) / 16);
+    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
+    return p.counters != nullptr && !p.direct && !p.balanced && items > resident;
+}
+inline int mfma_work_mode(const SplitParams& p) { return p.balanced ? WM_SHARES : mfma_runs_as_queue(p) ? WM_QUEUE : WM_ONE; }
+
+// (MODE must be mfma_work_mode(p_in): the translation units of the modes instantiate one each, see launch_mfma_d)
+template <int QDT, bool FP8, int D, bool PROBE = false, int MODE = WM_ONE>
 int launch_pm(const SplitParams& p_in, hipStream_t stream) {
+    if (mfma_work_mode(p_in) != MODE) return (int)hipErrorInvalidValue;
     constexpr int kScratch = 4 * kTile * D;
     SplitParams p = p_in;
     p.head_tiles = (p.group + 15) / 16;
@@ -978,15 +1032,16 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     else if (p.page_size % RPL == 0) pm = PM_LOAD;
     else pm = PM_LANE;
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
-    // Persistent mode (work queue) whenever the KV range is split and the caller provided counters: items of a
-    // ragged batch differ in length, and a queue keeps every compute unit busy until the end.
     const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
-    p.persistent = (p.counters != nullptr && !p.direct && !p.balanced && p.total_items > resident) ? 1 : 0;
+    p.persistent = MODE == WM_QUEUE ? 1 : 0;
     const unsigned units = (unsigned)(p.hg_blocks * p.head_tiles);
     const dim3 grid = p.balanced ? dim3(units, (unsigned)p.workgroups / units)
                     : p.persistent ? dim3((unsigned)resident)
                                    : dim3(units, (unsigned)p.num_splits, (unsigned)p.batch);
     const dim3 block(64 * nw);
+    p.shares = (int32_t)grid.y;
+    p.grid_x = (int32_t)grid.x;
+    p.wavefronts = nw;
     // Register buffers per wavefront (tiles of loads that can be under way while a tile is worked on): two, or
     // one for the widest rows (two would not leave room for two workgroups per compute unit), in a single pass
     // whose wavefronts together hold 32 KB with one, and for long pieces with wave-uniform page numbers (equal
@@ -1001,7 +1056,7 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
     const bool one_buffer = D > 128 || (p.tune_buffers ? p.tune_buffers == 1
                                                        : ((shaped && kTileBytes * nw >= 32768 && !wide_fp8) || long_pieces));
 #define FDK_MFMA_LAUNCH(PMV, NB) \
-    hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE>), grid, block, lds_bytes, stream, p)
+    hipLaunchKernelGGL((splitkv_mfma_kernel<QDT, FP8, PMV, NB, D, PROBE, MODE>), grid, block, lds_bytes, stream, p)
 #define FDK_MFMA_LAUNCH_PM(NB)                                    \
     switch (pm) {                                                 \
         case PM_TILE: FDK_MFMA_LAUNCH(PM_TILE, NB); break;        \
@@ -1020,12 +1075,12 @@ int launch_pm(const SplitParams& p_in, hipStream_t stream) {
 }
 
 
-template <int D>
+template <int D, int MODE>
 int launch_mfma_d(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
     const bool fp8 = kv_dtype == FDK_FP8_E4M3;
     if (q_dtype == FDK_BF16)
-        return fp8 ? launch_pm<FDK_BF16, true, D>(p, stream) : launch_pm<FDK_BF16, false, D>(p, stream);
-    return fp8 ? launch_pm<FDK_FP16, true, D>(p, stream) : launch_pm<FDK_FP16, false, D>(p, stream);
+        return fp8 ? launch_pm<FDK_BF16, true, D, false, MODE>(p, stream) : launch_pm<FDK_BF16, false, D, false, MODE>(p, stream);
+    return fp8 ? launch_pm<FDK_FP16, true, D, false, MODE>(p, stream) : launch_pm<FDK_FP16, false, D, false, MODE>(p, stream);
 }
 
 }  // namespace

@@ -4,9 +4,21 @@
 
 namespace fdk {
 
-int launch_splitkv_mfma_d64(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
-int launch_splitkv_mfma_d128(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
-int launch_splitkv_mfma_d256(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
+#define FDK_DECLARE_MFMA(D)                                                                                   \
+    int launch_splitkv_mfma_d##D(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);        \
+    int launch_splitkv_mfma_d##D##_queue(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream); \
+    int launch_splitkv_mfma_d##D##_bal(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream);
+FDK_DECLARE_MFMA(64)
+FDK_DECLARE_MFMA(128)
+FDK_DECLARE_MFMA(256)
+#undef FDK_DECLARE_MFMA
+// (the same rule as mfma_work_mode in the kernel header, which this file does not include)
+static int work_mode_of(const SplitParams& p) {
+    const int hg_per_wg = (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) ? 1 : p.hg_per_wg;
+    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + 15) / 16);
+    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);
+    return p.balanced ? 2 : (p.counters != nullptr && !p.direct && items > resident) ? 1 : 0;
+}
 
 bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim) {
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
@@ -40,12 +52,20 @@ int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg) {
 
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
     if (p.probe) return launch_splitkv_mfma_probe(p, kv_dtype, stream);
+    // the ways of handing out pieces are kernels of their own, instantiated in translation units of their own
+    const int mode = work_mode_of(p);
+#define FDK_MFMA_CASE(D)                                                                        \
+    case D:                                                                                     \
+        return mode == 2 ? launch_splitkv_mfma_d##D##_bal(p, q_dtype, kv_dtype, stream)         \
+             : mode == 1 ? launch_splitkv_mfma_d##D##_queue(p, q_dtype, kv_dtype, stream)       \
+                         : launch_splitkv_mfma_d##D(p, q_dtype, kv_dtype, stream);
     switch (p.head_dim) {
-        case 64: return launch_splitkv_mfma_d64(p, q_dtype, kv_dtype, stream);
-        case 128: return launch_splitkv_mfma_d128(p, q_dtype, kv_dtype, stream);
-        case 256: return launch_splitkv_mfma_d256(p, q_dtype, kv_dtype, stream);
+        FDK_MFMA_CASE(64)
+        FDK_MFMA_CASE(128)
+        FDK_MFMA_CASE(256)
         default: return (int)hipErrorInvalidValue;
     }
+#undef FDK_MFMA_CASE
 }
 
 }  // namespace fdk

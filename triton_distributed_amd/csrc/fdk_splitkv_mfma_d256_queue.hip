@@ -1,0 +1,10 @@
+// Matrix-core split-KV kernels for head_dim = 256: per-sequence chunks pulled from a work queue.
+#include "fdk_splitkv_mfma.h"
+
+namespace fdk {
+
+int launch_splitkv_mfma_d256_queue(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    return launch_mfma_d<256, WM_QUEUE>(p, q_dtype, kv_dtype, stream);
+}
+
+}  // namespace fdk

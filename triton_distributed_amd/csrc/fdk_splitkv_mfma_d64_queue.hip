@@ -1,0 +1,10 @@
+// Matrix-core split-KV kernels for head_dim = 64: per-sequence chunks pulled from a work queue.
+#include "fdk_splitkv_mfma.h"
+
+namespace fdk {
+
+int launch_splitkv_mfma_d64_queue(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    return launch_mfma_d<64, WM_QUEUE>(p, q_dtype, kv_dtype, stream);
+}
+
+}  // namespace fdk

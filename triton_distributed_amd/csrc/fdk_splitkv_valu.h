@@ -70,7 +70,7 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nw = blockDim.x >> 6;
+    const int nw = p.wavefronts;                    // (= blockDim.x / 64; see SplitParams)
     const int piece = lane % LPR;
     const int lgrp = lane / LPR;
     const int hh = lgrp % HS;                       // kv head within the head group
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(512) void splitkv_valu_kernel(const SplitParams p) 
     if (c_start >= kv_len) {
         if (p.direct) {   // kv_len == 0 with a single split: defined result, no combine follows
             const int kv_heads_here = nhg * HS;
-            for (int idx = threadIdx.x; idx < kv_heads_here * heads_here * kHeadDim; idx += blockDim.x) {
+            for (int idx = threadIdx.x; idx < kv_heads_here * heads_here * kHeadDim; idx += 64 * nw) {
                 const int d = idx % kHeadDim, g = (idx / kHeadDim) % heads_here, kh = idx / (kHeadDim * heads_here);
                 const int hq = (hgb * kv_heads_here + kh) * p.group + ht * GT + g;
                 store_out(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d, 0.f, p.out_dtype);

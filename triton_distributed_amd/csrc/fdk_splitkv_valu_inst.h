@@ -8,9 +8,12 @@ namespace fdk {
 namespace valu {
 
 template <int QDT, bool FP8, int GT, int HS>
-int launch_pm(const SplitParams& p, const ValuGeometry& geo, int pm, hipStream_t stream) {
+int launch_pm(const SplitParams& p_in, const ValuGeometry& geo, int pm, hipStream_t stream) {
+    SplitParams p = p_in;
     const dim3 grid((unsigned)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles));
     const dim3 block(64 * geo.nwaves);
+    p.wavefronts = geo.nwaves;
+    p.grid_x = (int32_t)grid.x;
     const size_t lds = (size_t)(2 * geo.nwaves + (geo.nwaves / 2) * kHeadDim) * HS * GT * sizeof(float);
     switch (pm) {
         case PM_TILE:
