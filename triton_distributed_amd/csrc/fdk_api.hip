@@ -74,7 +74,7 @@ constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and n
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
 constexpr int kMinRaggedLen = 2048;      // shorter contexts: a single pass that fills the compute units stays
-constexpr int64_t kPieceOverheadBytes = 72 << 10;   // balanced mode: see piece_cost_granules
+constexpr int64_t kPieceOverheadBytes = 128 << 10;  // balanced mode: see piece_cost_granules
 constexpr double kStreamBytesPerUs = 6.5e6;   // what a well-filled split kernel streams (plan estimates only)
 constexpr double kSplitOverheadUs = 7.0;      // partial rows + combine launch of a split plan (plan estimates only)
 
@@ -392,13 +392,16 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     return FDK_OK;
 }
 
-// Balanced mode: what starting one more sequence costs a workgroup, in granules of the partition.  The fixed
-// time of a piece (table and q loads before its first rows, the merge of the wavefronts after its last) is
-// what a workgroup needs to stream about kPieceOverheadBytes.
+// Balanced mode: what a sequence boundary inside a share costs its workgroup, in granules of the partition.  The
+// fixed time of a piece (table and q loads before its first rows, the merge of the wavefronts after its last) is
+// what a workgroup needs to stream about kPieceOverheadBytes (measured on ragged batches of 16 and 64 sequences with
+// one and eight kv heads: 0 / 48 / 96 / 144 / 192 KB give 90.7 / 88.3 / 88.3 / 87.4 / 88.9, 165.7 / 164.0 / 162.3 /
+// 162.5 / 163.6 and 30.8 / 30.4 / 28.8 / 28.3 / 28.4 us per call).
 int piece_cost_granules(const fdk_decode_args* a, int kv_heads_per_wg) {
     const int64_t granule_bytes = (int64_t)fdk::kBalanceGranule * kv_heads_per_wg * 2 * a->head_dim * elem_size(a->kv_dtype);
-    const int64_t c = (kPieceOverheadBytes + granule_bytes / 2) / granule_bytes;
-    return (int)(c > 16 ? 16 : c);
+    // an even number: the kernel puts half of it in front of a sequence's tokens and half behind
+    const int64_t c = 2 * ((kPieceOverheadBytes + granule_bytes) / (2 * granule_bytes));
+    return (int)(c > 64 ? 64 : c);
 }
 
 // q-head tiles per kv head, as the resolved algorithm's kernel counts them
