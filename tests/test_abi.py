@@ -386,6 +386,15 @@ def test_plan_scales_splits_with_occupancy():
     rows = (shares + 4) * units * p_long.kv_heads_per_wg * 8           # group = 8 heads per tile
     assert p_long.num_splits * 4 * 64 >= rows > (p_long.num_splits - 1) * 4 * 64
     assert shares * p_long.chunk_tokens >= 4 * 131072                   # the shares cover every sequence
+    # ... but only where streaming the cache at its bound takes some tens of microseconds: a batch of the same kind with
+    # 8192-token tables (4 x 8192 x 8 heads x 512 B = 134 MB, about 20 us) is cut into chunks of each sequence's own
+    # length, one workgroup per compute unit; equal shares can still be forced for measurements
+    short_kw = dict(batch=4, num_q_heads=64, page_size=64, max_pages=128, table_stride_b=128, q_stride_b=64 * 128,
+                    out_stride_b=64 * 128, lse_stride_b=64)
+    p_mid = _plan(_args(**short_kw))
+    assert p_mid.balanced == 0 and p_mid.chunk_floor == 64 and p_mid.num_splits * 4 * (8 // p_mid.kv_heads_per_wg) == 256
+    assert _plan(_measured(dict(force_balanced=1), **short_kw)).balanced == 1
+    assert _decode_rc(_measured(dict(force_balanced=2), **short_kw)) == _lib.FDK_ESHAPE
     # a single sequence has nothing to balance: per-sequence chunks that follow its own length
     p_one = _plan(_args(batch=1, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
                         q_stride_b=64 * 128, out_stride_b=64 * 128, lse_stride_b=64))

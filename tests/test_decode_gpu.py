@@ -664,7 +664,7 @@ def test_hip_graph_replays_follow_the_inputs(cuda_device, mode):
     elif mode == "chunks_queue":
         b, hq, hkv, n_max, kw = 12, 32, 8, 3000, dict(kv_split=24)        # 12*24*4 items > 512 resident workgroups
     else:
-        b, hq, hkv, n_max, kw = 3, 8, 1, 40000, {}
+        b, hq, hkv, n_max, kw = 3, 8, 1, 40000, dict(force_balanced=True)    # (a batch this small is cut into chunks otherwise)
     d, page = 128, 16
     pages = (n_max + page - 1) // page
     pool = b * pages
@@ -1042,9 +1042,12 @@ def test_balanced_mode_ragged_batches(cuda_device, name):
         v, vs = wl.quantize_kv_fp8(v)
         ref_kv = (ofp8.dequant_per_head(k, ks), ofp8.dequant_per_head(v, vs))
     scale = d ** -0.5
-    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens))
+    # (equal shares are the planner's own choice only for batches that stream for some tens of microseconds; these
+    # small ones force them)
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens), force_balanced=True)
     assert plan.balanced and plan.workgroups > 0, plan
-    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=max(lens), k_scale=ks, v_scale=vs)
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=max(lens), k_scale=ks, v_scale=vs,
+                                force_balanced=True)
     # chunk mode on the same inputs (a forced split count)
     out_c, lse_c = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=max(lens), k_scale=ks, v_scale=vs,
                                     kv_split=7)
@@ -1079,12 +1082,13 @@ def test_balanced_mode_with_soft_cap_strides_and_output_forms(cuda_device):
     table = table.to(cuda_device)
     lens_t = _lens_t(lens, cuda_device)
     scale, cap = d ** -0.5, 30.0
-    assert tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens)).balanced
+    assert tda.get_split_kv_plan(q, k, v, table, lens_t, max_kv_len=max(lens), force_balanced=True).balanced
     out32 = torch.full((3, hq, d + 3), float("nan"), dtype=torch.float32, device=cuda_device)
-    o, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), out=out32[:, :, :d])
+    o, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), out=out32[:, :, :d],
+                              force_balanced=True)
     packed = torch.full((3, hq, d + 1), float("nan"), dtype=torch.float16, device=cuda_device)
     tda.prepare_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), packed_out=packed,
-                       want_lse=False).run()
+                       want_lse=False, force_balanced=True).run()
     torch.cuda.synchronize()
     assert o.data_ptr() == out32.data_ptr() and torch.isnan(out32[:, :, d:]).all()      # nothing written past D
     o64, l64 = cf.attn_fp64(q, k, v, table, lens, scale, cap)
@@ -1111,8 +1115,8 @@ def test_balanced_mode_clamps_lengths_like_the_other_modes(cuda_device):
     table[2, :1875] = perm[width:width + 1875]
     table = table.to(cuda_device)
     lens_t = _lens_t([cap + 1000, -1, 30000], cuda_device)
-    assert tda.get_split_kv_plan(q, k, v, table, lens_t).balanced
-    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5)
+    assert tda.get_split_kv_plan(q, k, v, table, lens_t, force_balanced=True).balanced
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, d ** -0.5, force_balanced=True)
     torch.cuda.synchronize()
     assert torch.all(out[1] == 0) and torch.all(torch.isneginf(lse[1]))
     _check(out[[0, 2]], lse[[0, 2]], q[[0, 2]], k, v, table[[0, 2]], [cap, 30000], d ** -0.5, tag="balanced clamp")
@@ -1647,7 +1651,8 @@ def test_single_launch_decode_against_the_oracle_and_the_two_launch_form(cuda_de
     k, v, table = k.to(cuda_device), v.to(cuda_device), table.to(cuda_device)
     lens_t = _lens_t(lens, cuda_device)
     scale = d ** -0.5
-    kw = dict(kv_split=kv_split, k_scale=ks, v_scale=vs, max_kv_len=max(max(lens), 1))
+    kw = dict(kv_split=kv_split, k_scale=ks, v_scale=vs, max_kv_len=max(max(lens), 1),
+              force_balanced=name.startswith("balanced"))
     two = tda.prepare_decode(q, k, v, table, lens_t, scale, work_queue=False, **kw)
     one = tda.prepare_decode(q, k, v, table, lens_t, scale, single_launch=True, **kw)
     assert one.plan.num_splits > 1 and one.args.counters and not two.args.counters, one.plan

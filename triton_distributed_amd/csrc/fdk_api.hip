@@ -74,6 +74,11 @@ constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and n
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
 constexpr int kMinRaggedLen = 2048;      // shorter contexts: a single pass that fills the compute units stays
+constexpr double kBalancedMinStreamUs = 48.0;   // batches that do not fill the compute units, lengths unknown: equal shares
+                                                // only if streaming the cache at its bound takes this long (below, chunks of
+                                                // each sequence's own length are 1-4 us faster whether the lengths turn out
+                                                // ragged or alike; above, equal shares win by 2-14 % on ragged batches and
+                                                // lose 2-5 % on uniform ones: bench.py --op plan-sweep)
 constexpr int64_t kPieceOverheadBytes = 128 << 10;  // balanced mode: see piece_cost_granules
 constexpr double kStreamBytesPerUs = 6.5e6;   // what a well-filled split kernel streams (plan estimates only)
 constexpr double kSplitOverheadUs = 7.0;      // partial rows + combine launch of a split plan (plan estimates only)
@@ -346,7 +351,8 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const bool uniform = alike && !rebalance && !underfilled && !force_balanced;
     // (a single sequence has nothing to balance: its own length in equal chunks, below, does the same without the
     // pass over kv_lens and with a combine that knows where its rows are - 27 us against 34 us for 32768 tokens)
-    if (algo == FDK_ALGO_MFMA && may_split && !uniform && batch > 1 && batch <= kMaxBalancedBatch &&
+    const bool long_enough = alike || rebalance || force_balanced || stream_us >= kBalancedMinStreamUs;
+    if (algo == FDK_ALGO_MFMA && may_split && !uniform && long_enough && batch > 1 && batch <= kMaxBalancedBatch &&
         columns < (1 << 30)) {                                            // the kernel counts granules in int32
         const int64_t gran = fdk::kBalanceGranule;
         int64_t shares = columns / (min_chunk / gran);

@@ -240,12 +240,18 @@ def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
 
 
 def get_split_kv_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale=1.0, soft_cap=0.0, kv_split=-1,
-                      max_kv_len=None, algo="auto", num_cus: int = 0, min_kv_len=None) -> SplitKvPlan:
-    """The split count / chunk length / algorithm a decode call with these tensors will use."""
+                      max_kv_len=None, algo="auto", num_cus: int = 0, min_kv_len=None, force_balanced=False) -> SplitKvPlan:
+    """The split count / chunk length / algorithm a decode call with these tensors will use (``force_balanced``: the
+    plan of ``prepare_decode(..., force_balanced=True)``, a measurement aid)."""
     a = _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len,
                    None, None, algo, check_device=False, min_kv_len=min_kv_len)
     if num_cus > 0:
         a.flags |= _lib.FDK_FLAG_DRY_RUN
+    if force_balanced:
+        measure = FdkMeasureArgs()
+        measure.struct_size = C.sizeof(FdkMeasureArgs)
+        measure.force_balanced = 1
+        a.measure = C.addressof(measure)
     return _plan_of(a, num_cus)
 
 
@@ -485,7 +491,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  v_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                  lse: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
                  algo: str = "auto", stream=None, min_kv_len: Optional[int] = None,
-                 fp8_fold_k_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+                 fp8_fold_k_scale: bool = False, force_balanced: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Local (one GPU's share) split-KV GQA decode attention over a paged KV cache.
 
     q            [B, Hq, D] bf16/fp16, one query token per sequence
@@ -505,6 +511,7 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  per-sequence chunks follow each sequence's own length; results never depend on it
     k_scale/v_scale  [Hkv] fp32 dequantisation scales of an fp8 cache
     fp8_fold_k_scale fp8 cache: apply k_scale to the logits instead of to every K value (see ``prepare_decode``)
+    force_balanced   measurement / test aid: equal shares of the whole batch whatever the planner would choose
 
     Returns ``(out [B,Hq,D] in q's dtype, lse [B,Hq] fp32)``: out is normalised by the local softmax sum
     and lse = ln sum exp(scaled logits) - what the cross-rank combine consumes."""
@@ -513,7 +520,8 @@ def flash_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     call = prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap=soft_cap,
                           kv_split=kv_split, max_kv_len=max_kv_len, k_scale=k_scale, v_scale=v_scale,
                           out=out, lse=lse, workspace=workspace, algo=algo, min_kv_len=min_kv_len,
-                          fp8_fold_k_scale=fp8_fold_k_scale, stream_scratch=stream if q.is_cuda else None,
+                          fp8_fold_k_scale=fp8_fold_k_scale, force_balanced=force_balanced,
+                          stream_scratch=stream if q.is_cuda else None,
                           work_queue=kv_split > 0)      # the library's own plans never exceed the resident set
     return call.run(stream)
 
