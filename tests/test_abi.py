@@ -374,8 +374,15 @@ def test_plan_scales_splits_with_occupancy():
                         q_stride_b=96 * 128, out_stride_b=96 * 128, lse_stride_b=96))
     assert p_ref.balanced == 0 and p_ref.chunk_tokens % 16 == 0 and p_ref.kv_heads_per_wg == 2
     assert 6 * p_ref.num_splits <= 256 < 6 * (p_ref.num_splits + 3)
-    p24 = _plan(_args(batch=24, max_pages=64, table_stride_b=64))       # 96 units, 1024 tokens
-    assert p24.balanced == 0 and p24.num_splits == 2 and p24.chunk_tokens == 512
+    # 96 units, 1024 tokens: one workgroup per compute unit where the host vouches for the lengths; lengths it knows
+    # nothing about get two (finer chunks of the long sequences, should the batch be ragged) once the cache streams for
+    # more than a dozen microseconds
+    p24 = _plan(_args(batch=24, max_pages=64, table_stride_b=64, max_kv_len=1024, min_kv_len=1024))
+    assert p24.balanced == 0 and p24.num_splits == 2 and p24.chunk_tokens == 512 and p24.chunk_floor == 0
+    p24u = _plan(_args(batch=24, max_pages=64, table_stride_b=64))
+    assert p24u.balanced == 0 and p24u.num_splits == 4 and p24u.chunk_tokens == 256 and p24u.chunk_floor == 64
+    p8u = _plan(_args(batch=8, max_pages=64, table_stride_b=64))        # 5 us of streaming: one per compute unit
+    assert p8u.balanced == 0 and p8u.num_splits == 8 and p8u.chunk_floor == 64
     # few units, long context: balanced mode - one workgroup per compute unit, they share the KV ranges of the whole
     # batch, each gets a long share, and the workspace holds (shares + batch) slots per head block
     p_long = _plan(_args(batch=4, num_q_heads=64, page_size=64, max_pages=2048, table_stride_b=2048,
@@ -388,11 +395,11 @@ def test_plan_scales_splits_with_occupancy():
     assert shares * p_long.chunk_tokens >= 4 * 131072                   # the shares cover every sequence
     # ... but only where streaming the cache at its bound takes some tens of microseconds: a batch of the same kind with
     # 8192-token tables (4 x 8192 x 8 heads x 512 B = 134 MB, about 20 us) is cut into chunks of each sequence's own
-    # length, one workgroup per compute unit; equal shares can still be forced for measurements
+    # length, two workgroups per compute unit (lengths unknown); equal shares can still be forced for measurements
     short_kw = dict(batch=4, num_q_heads=64, page_size=64, max_pages=128, table_stride_b=128, q_stride_b=64 * 128,
                     out_stride_b=64 * 128, lse_stride_b=64)
     p_mid = _plan(_args(**short_kw))
-    assert p_mid.balanced == 0 and p_mid.chunk_floor == 64 and p_mid.num_splits * 4 * (8 // p_mid.kv_heads_per_wg) == 256
+    assert p_mid.balanced == 0 and p_mid.chunk_floor == 64 and p_mid.num_splits * 4 * (8 // p_mid.kv_heads_per_wg) == 512
     assert _plan(_measured(dict(force_balanced=1), **short_kw)).balanced == 1
     assert _decode_rc(_measured(dict(force_balanced=2), **short_kw)) == _lib.FDK_ESHAPE
     # a single sequence has nothing to balance: per-sequence chunks that follow its own length

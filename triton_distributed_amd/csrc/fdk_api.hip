@@ -74,7 +74,8 @@ constexpr int kDryRunCus = 256;           // a dry run plans for an MI355X and n
 constexpr int kMaxBalancedBatch = 512;   // balanced mode: every wavefront scans kv_lens, keep that short
 constexpr int kMinBalancedShare = 512;   // balanced mode only if a workgroup's share has this many tokens
 constexpr int kMinRaggedLen = 2048;      // shorter contexts: a single pass that fills the compute units stays
-constexpr double kBalancedMinStreamUs = 48.0;   // batches that do not fill the compute units, lengths unknown: equal shares
+constexpr double kFinerChunksStreamUs = 12.0;   // see make_plan
+constexpr double kBalancedMinStreamUs = 40.0;   // batches that do not fill the compute units, lengths unknown: equal shares
                                                 // only if streaming the cache at its bound takes this long (below, chunks of
                                                 // each sequence's own length are 1-4 us faster whether the lengths turn out
                                                 // ragged or alike; above, equal shares win by 2-14 % on ragged batches and
@@ -324,6 +325,11 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         splits = a->num_splits;
     } else if (may_split && !rebalance) {
         splits = (int64_t)num_cus / units;
+        // Lengths the host does not vouch for, and enough to stream that the start of a workgroup is not what counts
+        // (kFinerChunksStreamUs): two workgroups per compute unit.  If the batch turns out ragged, the chunks of its long
+        // sequences are what the call waits for, and finer ones end up to 10 % sooner; if it turns out uniform, the
+        // second workgroup per unit costs 1-3 %.
+        if (!alike && algo == FDK_ALGO_MFMA && batch > 1 && stream_us >= kFinerChunksStreamUs) splits *= 2;
         if (splits > most_chunks) splits = most_chunks;
     }
     memset(plan, 0, sizeof(*plan));
