@@ -234,7 +234,7 @@ def _placed(args, tda, pools):
         return pools
     out = []
     for k, v in pools:
-        k2, v2 = tda.alloc_kv_pools(tuple(k.shape), k.dtype, k.device, zero=False)
+        k2, v2 = tda.alloc_kv_pools(tuple(k.shape), k.dtype, k.device, zero=False, v_shape=tuple(v.shape))
         k2.copy_(k)
         v2.copy_(v)
         out.append((k2, v2))
@@ -521,7 +521,7 @@ def main():
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
     inp = inp_cpu.to(dev)
     pools = [(inp.k_cache, inp.v_cache)]
-    pool_bytes = 2 * inp.k_cache.numel() * inp.k_cache.element_size()
+    pool_bytes = (inp.k_cache.numel() + inp.v_cache.numel()) * inp.k_cache.element_size()
     rotate = max(1, args.rotate)
     if args.rotate > 1:
         rotate = max(rotate, min(16, -(-(1 << 30) // max(pool_bytes, 1))))       # small pools: more of them
@@ -532,8 +532,8 @@ def main():
             mk = lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
                 torch.float8_e4m3fn)
         else:
-            mk = lambda: torch.randn(inp.k_cache.shape, generator=g, device=dev, dtype=inp.k_cache.dtype)
-        pools.append((mk(), mk()))
+            mk = lambda like=inp.k_cache: torch.randn(like.shape, generator=g, device=dev, dtype=like.dtype)
+        pools.append((mk(), mk(inp.v_cache) if inp.cfg.kv_dtype != "fp8_e4m3" else mk()))
     def prepare_all(pp):
         return [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                    v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,
@@ -699,7 +699,7 @@ def main():
     # kv_split = 32 (sp_flash_decode_layer.py:62,100-110), output_combine given; fp8 caches are not part of that signature
     ref_entry_us = ref_entry_fb_us = cold_fb_us = None
     if inp.cfg.kv_dtype != "fp8_e4m3" and not args.kernel_only:
-        oc = torch.empty((inp.q.shape[0], inp.q.shape[1], inp.q.shape[2] + 1), dtype=inp.q.dtype, device=dev)
+        oc = torch.empty((inp.q.shape[0], inp.q.shape[1], inp.v_cache.shape[-1] + 1), dtype=inp.q.dtype, device=dev)
         ref_call = lambda i: tda.gqa_fwd_batch_decode_intra_rank(inp.q, *pools[i % len(pools)], None, None, inp.kv_lens,
                                                                  inp.block_table, inp.sm_scale, output_combine=oc, kv_split=32)
         ref_entry_us = timed_loop(ref_call, n_entry)

@@ -593,3 +593,63 @@ def test_single_launch_flag_needs_counters_to_take_effect():
     n = lib.fdk_counters_len(C.byref(_args(batch=4)))
     assert _decode_rc(_args(batch=4, flags=fl, counters=0x90000, counters_len=n)) == 0
     assert _decode_rc(_args(batch=4, flags=fl, counters=0x90000, counters_len=n - 1)) == _lib.FDK_EWORKSPACE
+
+
+def _dims(dk, dv, **kw):
+    """The block of _args with q / K rows of dk values and V / output rows of dv (v_head_dim; 0 where they are alike)."""
+    base = dict(head_dim=dk, v_head_dim=0 if dv == dk else dv, q_stride_b=32 * dk, q_stride_h=dk,
+                k_stride_page=16 * 8 * dk, k_stride_tok=8 * dk, k_stride_head=dk,
+                v_stride_page=16 * 8 * dv, v_stride_tok=8 * dv, v_stride_head=dv,
+                out_stride_b=32 * dv, out_stride_h=dv, sm_scale=dk ** -0.5)
+    base.update(kw)
+    return _args(**base)
+
+
+def test_head_dims_of_two_segments_and_v_rows_of_their_own_length():
+    # the reference's BLOCK_HEAD_DIM + BLOCK_DPE and V_DIM (flash_decode.py:103-109): 192 = 128 + 64, 576 = 512 + 64
+    lib = _lib.load()
+    for dk, dv in ((192, 192), (192, 128), (576, 512), (128, 128), (64, 64), (256, 256)):
+        assert _decode_rc(_dims(dk, dv)) == 0, (dk, dv, lib.fdk_last_error())
+    assert _decode_rc(_args(v_head_dim=128)) == 0                       # spelled out, equal to head_dim
+    for dk, dv in ((192, 64), (128, 64), (576, 576), (256, 128), (96, 96), (512, 512), (576, 192)):
+        assert _decode_rc(_dims(dk, dv)) == _lib.FDK_EUNSUPPORTED, (dk, dv)
+    assert _decode_rc(_args(v_head_dim=-1)) == _lib.FDK_ESHAPE
+    # what follows v_head_dim: the output row (and the packed row), the V head stride, the workspace
+    assert _decode_rc(_dims(192, 128, out_stride_h=127)) == _lib.FDK_ESHAPE
+    assert _decode_rc(_dims(192, 128, flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE)) == _lib.FDK_ESHAPE
+    assert _decode_rc(_dims(192, 128, flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_PACK_LSE, out_stride_h=129,
+                            out_stride_b=32 * 129)) == 0
+    assert _decode_rc(_dims(192, 128, v_stride_head=64)) == _lib.FDK_ESHAPE
+    a = _dims(576, 512, batch=4, max_kv_len=8192)
+    p = _plan(a)
+    assert p.num_splits > 1
+    need = lib.fdk_workspace_bytes(4, 32, 512, p.num_splits)
+    a.workspace_bytes = need
+    assert _decode_rc(a) == 0
+    a.workspace_bytes = need - 1
+    assert _decode_rc(a) == _lib.FDK_EWORKSPACE
+    # built for 16-bit caches on the matrix-core path, without the single-launch form
+    assert _decode_rc(_dims(192, 192, kv_dtype=_lib.FDK_FP8_E4M3)) == _lib.FDK_EUNSUPPORTED
+    assert _decode_rc(_dims(192, 192, algo=_lib.FDK_ALGO_VALU)) == _lib.FDK_EUNSUPPORTED
+    assert _decode_rc(_dims(192, 192, flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_SINGLE_LAUNCH)) == _lib.FDK_EUNSUPPORTED
+    assert _plan(_dims(192, 128)).algo == _lib.FDK_ALGO_MFMA
+    # a caller of the revision before v_head_dim existed: the field reads as zero
+    old = _dims(192, 128)
+    old.struct_size = FdkDecodeArgs.v_head_dim.offset
+    assert _decode_rc(old) == _lib.FDK_ESHAPE              # V strides of 128-value rows are too short for 192-value rows
+    old = _args()
+    old.struct_size = FdkDecodeArgs.v_head_dim.offset
+    assert _decode_rc(old) == 0
+
+
+def test_plans_of_wide_rows_keep_to_what_a_compute_unit_holds():
+    # blocks of 4 or 8 kv heads are eight wavefronts; rows of more than 512 values per token and kv head (K and V
+    # together) leave registers and LDS for four, i.e. at most two heads per workgroup
+    big = dict(batch=512, max_kv_len=2048, min_kv_len=2048)
+    assert _plan(_dims(192, 192, **big)).kv_heads_per_wg == 8
+    assert _plan(_dims(192, 128, **big)).kv_heads_per_wg == 8
+    p = _plan(_dims(576, 512, **big))
+    assert p.kv_heads_per_wg == 2 and p.num_splits == 1
+    # streaming estimates count the K and the V row: a (192, 128) cache streams 5/6 of what a (192, 192) cache does
+    a, b = _plan(_dims(192, 192, batch=8, max_kv_len=4096)), _plan(_dims(192, 128, batch=8, max_kv_len=4096))
+    assert a.num_splits >= 1 and b.num_splits >= 1

@@ -207,6 +207,169 @@ def test_other_head_sizes_fp8_pages_and_rank_merge(cuda_device, head_size, page)
     torch.testing.assert_close(lse_m, l2 + math.log(2.0), atol=1e-4, rtol=0)
 
 
+# ---- q / K rows of two segments and V rows of their own length: the reference's BLOCK_HEAD_DIM + BLOCK_DPE and V_DIM
+# (flash_decode.py:103-109,187-191,210-214): 192 = 128 + 64 with V rows of 192 or 128, 576 = 512 + 64 with V rows of 512 ----
+TWO_SEGMENT_DIMS = [(192, 192), (192, 128), (576, 512)]
+
+
+def _two_segment_inputs(device, dims, lens, heads, page, dtype, seed, spare_pages=3, table_extra=0):
+    """q [B,Hq,Dk], K pool [pages,P,Hkv,Dk], V pool [pages,P,Hkv,Dv], a table of distinct pages in random order (columns
+    past a sequence's pages point at a page of NaN), lengths."""
+    dk, dv = dims
+    hq, hkv = heads
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    per_seq = [(n + page - 1) // page for n in lens]
+    width = max(max(per_seq), 1) + table_extra
+    n_pages = sum(per_seq) + spare_pages + 1
+    q = torch.randn(len(lens), hq, dk, generator=g).to(dtype).to(device)
+    k = torch.randn(n_pages, page, hkv, dk, generator=g).to(dtype).to(device)
+    v = torch.randn(n_pages, page, hkv, dv, generator=g).to(dtype).to(device)
+    k[n_pages - 1] = float("nan")
+    v[n_pages - 1] = float("nan")
+    perm = torch.randperm(n_pages - 1, generator=g).to(torch.int32)
+    table = torch.full((len(lens), width), n_pages - 1, dtype=torch.int32)
+    at = 0
+    for b, n in enumerate(per_seq):
+        table[b, :n] = perm[at:at + n]
+        at += n
+    return q, k, v, table.to(device), _lens_t(lens, device)
+
+
+@pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
+@pytest.mark.parametrize("kv_lens", [[1320, 18, 463], [1, 54, 293, 70]])
+@pytest.mark.parametrize("num_heads", [(16, 16), (32, 8), (64, 8), (6, 1)])
+@pytest.mark.parametrize("block_size", [1, 16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("soft_cap", [0, 50])
+def test_reference_grid_two_segment_head_dims(cuda_device, dims, kv_lens, num_heads, block_size, dtype, soft_cap):
+    print(f"case dims={dims} lens={kv_lens} heads={num_heads} P={block_size} {dtype} cap={soft_cap}", flush=True)
+    dk, dv = dims
+    num_blocks = 256
+    g = torch.Generator(device="cpu").manual_seed(hash((dims, tuple(kv_lens), num_heads, block_size)) & 0xFFFF)
+    hq, hkv = num_heads
+    scale = dk ** -0.5
+    q = torch.randn(len(kv_lens), hq, dk, generator=g).to(dtype).to(cuda_device)
+    k = torch.randn(num_blocks + 1, block_size, hkv, dk, generator=g).to(dtype).to(cuda_device)
+    v = torch.randn(num_blocks + 1, block_size, hkv, dv, generator=g).to(dtype).to(cuda_device)
+    max_blocks = (max(kv_lens) + block_size - 1) // block_size
+    table = torch.randint(0, num_blocks, (len(kv_lens), max_blocks), generator=g, dtype=torch.int32).to(cuda_device)
+    lens_t = _lens_t(kv_lens, cuda_device)
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap))
+    out1, lse1 = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap), kv_split=1)
+    out9, lse9 = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=float(soft_cap), kv_split=9)
+    o2 = tda.gqa_fwd_batch_decode(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale, float(soft_cap))
+    packed = tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, [1] * len(kv_lens), lens_t, table, scale,
+                                                 float(soft_cap), kv_split=32)
+    torch.cuda.synchronize()
+    assert out.shape == (len(kv_lens), hq, dv) and out.dtype == dtype
+    for o, l, tag in ((out, lse, "auto"), (out1, lse1, "S=1"), (out9, lse9, "S=9")):
+        _check(o, l, q, k, v, table, kv_lens, scale, float(soft_cap), tag=f"dims={dims} {tag}")
+    assert torch.equal(o2, out)
+    assert packed.shape == (len(kv_lens), hq, dv + 1) and packed.dtype == dtype
+    torch.testing.assert_close(packed[..., :dv].float(), out.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(packed[..., dv].float(), lse, atol=3e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
+@pytest.mark.parametrize("page", [16, 64, 4, 6, 1])
+def test_two_segment_head_dims_in_every_plan(cuda_device, dims, page):
+    """Ragged batches through equal shares, own-length chunks, the work queue and a single pass; page sizes whose page
+    numbers come one per tile (16, 64) and one per row (4, 6, 1); empty sequences; fp32 output; the rank merge."""
+    dk, dv = dims
+    scale = dk ** -0.5
+    g = torch.Generator().manual_seed(dk + dv + page)
+    lens = [int(x) for x in torch.randint(1, 3000, (12,), generator=g)]
+    lens[3], lens[7] = 0, 1
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, (16, 2), page, torch.bfloat16, 77 + page, table_extra=2)
+    ref_plan = tda.get_split_kv_plan(q, k, v, table, lens_t, scale)
+    assert ref_plan.algo == "mfma"
+    live = [i for i, n in enumerate(lens) if n > 0]
+
+    def check(o, l, tag):
+        assert torch.isfinite(o.float()).all() and float(o[3].abs().max()) == 0 and bool((l[3] == -math.inf).all()), tag
+        _check(o[live], l[live], q[live], k, v, table[live], [lens[i] for i in live], scale, tag=f"dims={dims} P={page} {tag}")
+
+    out_b, lse_b = tda.flash_decode(q, k, v, table, lens_t, scale, force_balanced=True)
+    plan_b = tda.get_split_kv_plan(q, k, v, table, lens_t, scale, force_balanced=True)
+    assert plan_b.balanced
+    out_c, lse_c = tda.flash_decode(q, k, v, table, lens_t, scale, kv_split=5)
+    out_q, lse_q = tda.flash_decode(q, k, v, table, lens_t, scale, kv_split=48)      # 12 x 48 pieces: more than are resident, a queue
+    out_f = torch.empty(len(lens), 16, dv, dtype=torch.float32, device=cuda_device)
+    _, lse_f = tda.flash_decode(q, k, v, table, lens_t, scale, out=out_f)
+    torch.cuda.synchronize()
+    check(out_b, lse_b, "equal shares")
+    check(out_c, lse_c, "5 chunks")
+    check(out_q, lse_q, "work queue")
+    check(out_f, lse_f, "fp32 out")
+    torch.testing.assert_close(out_f, out_b.float(), atol=1e-2, rtol=1e-2)
+    # a batch that fills the GPU by itself: whole sequences per workgroup, in blocks of kv heads (at most two heads per
+    # workgroup where a token's K and V rows hold more than 512 values)
+    lens2 = [int(x) for x in torch.randint(40, 160, (130,), generator=g)]
+    q2, k2, v2, table2, lens2_t = _two_segment_inputs(cuda_device, dims, lens2, (16, 8), page, torch.float16, 99 + page)
+    plan2 = tda.get_split_kv_plan(q2, k2, v2, table2, lens2_t, scale, max_kv_len=max(lens2), min_kv_len=max(lens2))
+    assert plan2.num_splits == 1 and plan2.kv_heads_per_wg == (2 if dk + dv > 512 else 4), plan2
+    o2, l2 = tda.flash_decode(q2, k2, v2, table2, lens2_t, scale, max_kv_len=max(lens2), min_kv_len=max(lens2))
+    torch.cuda.synchronize()
+    _check(o2, l2, q2, k2, v2, table2, lens2, scale, tag=f"dims={dims} P={page} single pass")
+    # the cross-rank merge on rows of dv values: a result merged with itself is itself, lse + ln 2
+    both = torch.stack([tda.pack_out_lse(o2, l2, torch.float32)] * 2)
+    lse_m = torch.empty_like(l2)
+    merged = tda.inter_rank_combine(both, lens2_t[None].repeat(2, 1), lse_out=lse_m)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(merged.float(), o2.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(lse_m, l2 + math.log(2.0), atol=1e-4, rtol=0)
+
+
+@pytest.mark.parametrize("seed", list(range(18)))
+def test_two_segment_head_dims_random_shapes(cuda_device, seed):
+    g = torch.Generator().manual_seed(4000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    dims = TWO_SEGMENT_DIMS[seed % 3]
+    hkv = [1, 2, 3, 4, 8][r(0, 4)]
+    group = [1, 2, 4, 7, 8, 16, 20][r(0, 6)]
+    page = [1, 2, 5, 8, 16, 32, 48, 128][r(0, 7)]
+    batch = r(1, 20)
+    top = [60, 700, 5000][r(0, 2)]
+    lens = [r(0 if batch > 1 else 1, top) for _ in range(batch)]
+    if max(lens) == 0:
+        lens[0] = 17
+    dtype = [torch.bfloat16, torch.float16][r(0, 1)]
+    cap = [0.0, 20.0][r(0, 1)]
+    split = [-1, -1, 1, 2, 7, 33][r(0, 5)]
+    hints = r(0, 1)
+    print(f"case seed={seed} dims={dims} heads=({hkv * group},{hkv}) P={page} B={batch} top={top} {dtype} cap={cap} "
+          f"split={split} hints={hints}", flush=True)
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, (hkv * group, hkv), page, dtype, 5000 + seed,
+                                                 table_extra=r(0, 3))
+    scale = dims[0] ** -0.5 * [1.0, 0.5, 2.0][r(0, 2)]
+    kw = dict(max_kv_len=max(lens), min_kv_len=min(lens)) if hints else {}
+    out, lse = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, kv_split=split, **kw)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    for i, n in enumerate(lens):
+        if n == 0:
+            assert float(out[i].abs().max()) == 0 and bool((lse[i] == -math.inf).all())
+    _check(out[live], lse[live], q[live], k, v, table[live], [lens[i] for i in live], scale, cap, tag=f"seed {seed}",
+           ref_tol=4e-2 if scale > dims[0] ** -0.5 else None)
+
+
+def test_what_is_not_built_for_two_segment_head_dims_is_refused(cuda_device):
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, (192, 128), [300, 20], (8, 2), 16, torch.bfloat16, 5)
+    with pytest.raises(ValueError, match="matrix-core"):
+        tda.flash_decode(q, k, v, table, lens_t, 1.0, algo="valu")
+    with pytest.raises(ValueError, match="single-launch"):
+        tda.prepare_decode(q, k, v, table, lens_t, 1.0, kv_split=4, single_launch=True).run()
+    k8, v8 = k.to(torch.float8_e4m3fn), v.to(torch.float8_e4m3fn)
+    with pytest.raises(ValueError, match="16-bit caches"):
+        tda.flash_decode(q, k8, v8, table, lens_t, 1.0)
+    for dk, dv in ((192, 64), (128, 64), (576, 576), (256, 128)):
+        qq = torch.zeros(2, 8, dk, dtype=torch.bfloat16, device=cuda_device)
+        kk = torch.zeros(8, 16, 2, dk, dtype=torch.bfloat16, device=cuda_device)
+        vv = torch.zeros(8, 16, 2, dv, dtype=torch.bfloat16, device=cuda_device)
+        with pytest.raises(ValueError, match="head_dim"):
+            tda.flash_decode(qq, kk, vv, table[:, :1], lens_t, 1.0)
+
+
 # ---- golden vectors and edge cases -----------------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["tiny", *EDGE_CASES])
 @pytest.mark.parametrize("kv_split", [-1, 1, 3, 32])

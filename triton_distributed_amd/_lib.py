@@ -12,7 +12,7 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libfdk.so"
 
 FDK_ABI_VERSION = 8
-FDK_ABI_REVISION = 1      # the library may be newer (its structs only grow at the end), never older
+FDK_ABI_REVISION = 2      # the library may be newer (its structs only grow at the end), never older
 
 # fdk_dtype
 FDK_BF16, FDK_FP16, FDK_FP8_E4M3, FDK_FP32 = 0, 1, 2, 3
@@ -62,6 +62,7 @@ class FdkDecodeArgs(C.Structure):
         ("length_feedback", C.c_void_p),
         ("reserved1", C.c_void_p), ("reserved2", C.c_int64),
         ("measure", C.c_void_p),           # FdkMeasureArgs*, null in product use
+        ("v_head_dim", C.c_int32), ("reserved3", C.c_int32),     # (revision 2) 0: V rows as long as q / K rows
     ]
 
 

@@ -31,6 +31,10 @@ SOURCES = [
     "fdk_splitkv_valu_fp16_fp8.hip", "fdk_splitkv_mfma_d64.hip", "fdk_splitkv_mfma_d128.hip", "fdk_splitkv_mfma_d256.hip",
     "fdk_splitkv_mfma_d64_bal.hip", "fdk_splitkv_mfma_d128_bal.hip", "fdk_splitkv_mfma_d256_bal.hip",
     "fdk_splitkv_mfma_d64_queue.hip", "fdk_splitkv_mfma_d128_queue.hip", "fdk_splitkv_mfma_d256_queue.hip", "fdk_kv_append.hip", "fdk_probe.hip",
+    # q / K rows of two segments (192 = 128 + 64, 576 = 512 + 64), V rows of their own length
+    "fdk_splitkv_mfma_d192.hip", "fdk_splitkv_mfma_d192_queue.hip", "fdk_splitkv_mfma_d192_bal.hip",
+    "fdk_splitkv_mfma_d192v128.hip", "fdk_splitkv_mfma_d192v128_queue.hip", "fdk_splitkv_mfma_d192v128_bal.hip",
+    "fdk_splitkv_mfma_d576v512.hip", "fdk_splitkv_mfma_d576v512_queue.hip", "fdk_splitkv_mfma_d576v512_bal.hip",
 ]
 
 # the translation units that contain the matrix-core split kernel: the only ones the timeline build compiles anew
@@ -79,7 +83,7 @@ def build(verbose: bool = True, jobs: int = 8, timeline: bool = False) -> Path:
             todo = [(src, obj) for src, obj in pairs if src.name in TIMELINE_SOURCES]
     if verbose:
         print(f"[fdk build] hipcc={hipcc} -> {lib_path}", flush=True)
-    todo = sorted(todo, key=lambda so: "splitkv_mfma_d" not in so[0].name)       # the longest compilations first
+    todo = sorted(todo, key=lambda so: so[0].name not in TIMELINE_SOURCES)       # the longest compilations first
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo)))) as ex:
         list(ex.map(lambda so: _compile_one(hipcc, so[0], so[1], extra), todo))
     tmp = lib_path.with_suffix(".so.tmp")

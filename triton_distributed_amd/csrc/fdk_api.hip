@@ -149,6 +149,14 @@ int adopt_call(const fdk_decode_args* args, Call* c) {
     return FDK_OK;
 }
 
+// values per V row / output row
+inline int v_dim(const fdk_decode_args* a) { return a->v_head_dim > 0 ? a->v_head_dim : a->head_dim; }
+// rows of one power-of-two segment, K and V alike: every path and option is built for them
+inline bool plain_dims(int dk, int dv) { return dk == dv && (dk == 64 || dk == 128 || dk == 256); }
+// rows of two segments (the reference's BLOCK_HEAD_DIM + BLOCK_DPE) and V rows shorter than K rows: matrix-core path,
+// 16-bit caches
+inline bool two_segment_dims(int dk, int dv) { return (dk == 192 && (dv == 192 || dv == 128)) || (dk == 576 && dv == 512); }
+
 // (a: a block in this library's layout, from adopt_call)
 int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) {
     if (a->batch < 0) return fail(FDK_ESHAPE, "batch %d < 0", a->batch);
@@ -156,8 +164,19 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         return fail(FDK_ESHAPE, "head counts must be positive (Hq=%d, Hkv=%d)", a->num_q_heads, a->num_kv_heads);
     if (a->num_q_heads % a->num_kv_heads != 0)
         return fail(FDK_ESHAPE, "Hq=%d not a multiple of Hkv=%d", a->num_q_heads, a->num_kv_heads);
-    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
-        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
+    if (a->v_head_dim < 0) return fail(FDK_ESHAPE, "v_head_dim %d < 0", a->v_head_dim);
+    const int dv = v_dim(a);
+    if (!plain_dims(a->head_dim, dv) && !two_segment_dims(a->head_dim, dv))
+        return fail(FDK_EUNSUPPORTED, "head_dim %d / v_head_dim %d not built (64, 128, 256; 192 with 192 or 128; 576 with 512)",
+                    a->head_dim, dv);
+    if (two_segment_dims(a->head_dim, dv)) {
+        if (a->kv_dtype != a->q_dtype)
+            return fail(FDK_EUNSUPPORTED, "head_dim %d / v_head_dim %d: built for 16-bit caches of the q dtype", a->head_dim, dv);
+        if (a->algo == FDK_ALGO_VALU)
+            return fail(FDK_EUNSUPPORTED, "head_dim %d / v_head_dim %d: built on the matrix-core path", a->head_dim, dv);
+        if (a->flags & FDK_FLAG_SINGLE_LAUNCH)
+            return fail(FDK_EUNSUPPORTED, "head_dim %d / v_head_dim %d: the single-launch form is not built", a->head_dim, dv);
+    }
     if (a->page_size <= 0) return fail(FDK_ESHAPE, "page_size %d <= 0", a->page_size);
     if (a->max_pages <= 0) return fail(FDK_ESHAPE, "max_pages %d <= 0", a->max_pages);
     // token positions, chunk bounds (start + chunk) and granule counts are 32-bit in the kernels
@@ -218,7 +237,7 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
     if (a->kv_dtype == FDK_FP8_E4M3 &&
         ((reinterpret_cast<uintptr_t>(a->k_scale) & 3u) || (reinterpret_cast<uintptr_t>(a->v_scale) & 3u)))
         return fail(FDK_EALIGN, "k_scale / v_scale must be 4-byte aligned");
-    if ((a->k_stride_head < a->head_dim || a->v_stride_head < a->head_dim) && a->num_kv_heads > 1)
+    if ((a->k_stride_head < a->head_dim || a->v_stride_head < dv) && a->num_kv_heads > 1)
         return fail(FDK_ESHAPE, "cache head stride < head_dim (k %lld, v %lld)", (long long)a->k_stride_head,
                     (long long)a->v_stride_head);
     if (a->table_stride_b < a->max_pages)
@@ -230,7 +249,7 @@ int validate(const fdk_decode_args* a, bool need_out, bool need_workspace_only) 
         if (a->out_dtype != FDK_BF16 && a->out_dtype != FDK_FP16 && a->out_dtype != FDK_FP32)
             return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);
         if (reinterpret_cast<uintptr_t>(a->out) % oes) return fail(FDK_EALIGN, "out not element aligned");
-        const int row = a->head_dim + ((a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0);
+        const int row = dv + ((a->flags & FDK_FLAG_PACK_LSE) ? 1 : 0);
         if (a->out_stride_h < row) return fail(FDK_ESHAPE, "out_stride_h %lld < %d", (long long)a->out_stride_h, row);
         if (a->lse && (reinterpret_cast<uintptr_t>(a->lse) & 3u)) return fail(FDK_EALIGN, "lse not 4-byte aligned");
         if (a->lse && a->lse_stride_b < a->num_q_heads)
@@ -246,12 +265,12 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     if (algo == FDK_ALGO_AUTO) {
         // The matrix-core path is the default for every group size: on MI355X it is at least as fast as the
         // vector path even for small groups, because it needs an order of magnitude fewer issue slots per KV byte.
-        algo = fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
+        algo = fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim, v_dim(a)) ? FDK_ALGO_MFMA : FDK_ALGO_VALU;
     }
-    if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim))
+    if (algo == FDK_ALGO_MFMA && !fdk::mfma_supported(a->q_dtype, a->kv_dtype, group, a->head_dim, v_dim(a)))
         return fail(FDK_EUNSUPPORTED, "MFMA path not built for q_dtype=%d kv_dtype=%d head_dim=%d", a->q_dtype,
                     a->kv_dtype, a->head_dim);
-    if (algo == FDK_ALGO_VALU && !fdk::valu_supported(a->q_dtype, a->kv_dtype, group, a->head_dim))
+    if (algo == FDK_ALGO_VALU && (v_dim(a) != a->head_dim || !fdk::valu_supported(a->q_dtype, a->kv_dtype, group, a->head_dim)))
         return fail(FDK_EUNSUPPORTED, "VALU path not built for q_dtype=%d kv_dtype=%d head_dim=%d (128 only)", a->q_dtype,
                     a->kv_dtype, a->head_dim);
 
@@ -266,7 +285,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     int kv_heads_per_wg = 1;
     int units_per_seq;
     if (algo == FDK_ALGO_MFMA) {
-        kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus);
+        kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus, a->head_dim + v_dim(a));
         units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg);
     } else {
         units_per_seq = fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
@@ -286,7 +305,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     //    pass runs at (fill + 1) / 2 of the even rate, fill = units / (rounds x compute units): 131 / 139 /
     //    159 us against 103 / 124 / 155 us of streaming time.
     const bool alike = a->min_kv_len > 0 && (int64_t)a->min_kv_len * 32 >= max_len * 31;
-    const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * 2.0 * a->head_dim *
+    const double stream_us = (double)batch * (double)max_len * a->num_kv_heads * (double)(a->head_dim + v_dim(a)) *
                              elem_size(a->kv_dtype) / kStreamBytesPerUs;      // what streaming the batch's cache takes
     bool rebalance = false;
     // (measurement aid: equal shares wherever they can run, to time them against the plan chosen here)
@@ -410,7 +429,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
 // one and eight kv heads: 0 / 48 / 96 / 144 / 192 KB give 90.7 / 88.3 / 88.3 / 87.4 / 88.9, 165.7 / 164.0 / 162.3 /
 // 162.5 / 163.6 and 30.8 / 30.4 / 28.8 / 28.3 / 28.4 us per call).
 int piece_cost_granules(const fdk_decode_args* a, int kv_heads_per_wg) {
-    const int64_t granule_bytes = (int64_t)fdk::kBalanceGranule * kv_heads_per_wg * 2 * a->head_dim * elem_size(a->kv_dtype);
+    const int64_t granule_bytes = (int64_t)fdk::kBalanceGranule * kv_heads_per_wg * (a->head_dim + v_dim(a)) * elem_size(a->kv_dtype);
     // an even number: the kernel puts half of it in front of a sequence's tokens and half behind
     const int64_t c = 2 * ((kPieceOverheadBytes + granule_bytes) / (2 * granule_bytes));
     return (int)(c > 64 ? 64 : c);
@@ -442,13 +461,13 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     float* part_lse = nullptr;
     int2* slot_desc = nullptr;           // one per (sequence, unit), behind the partial rows
     if (!direct && a->batch > 0) {
-        const size_t need = fdk_workspace_bytes(a->batch, a->num_q_heads, a->head_dim, S);
+        const size_t need = fdk_workspace_bytes(a->batch, a->num_q_heads, v_dim(a), S);
         if (!a->workspace) return fail(FDK_EWORKSPACE, "workspace is null; %zu bytes needed", need);
         if (!aligned16(a->workspace)) return fail(FDK_EALIGN, "workspace must be 16-byte aligned");
         if (a->workspace_bytes < need)
             return fail(FDK_EWORKSPACE, "workspace has %zu bytes; %zu needed for %d splits", a->workspace_bytes, need, S);
         part_o = reinterpret_cast<float*>(a->workspace);
-        part_lse = part_o + rows * S * a->head_dim;
+        part_lse = part_o + rows * S * v_dim(a);
         slot_desc = reinterpret_cast<int2*>((reinterpret_cast<uintptr_t>(part_lse + rows * S) + 7) & ~uintptr_t(7));
     }
     fdk::SplitParams& sp = r->sp;
@@ -468,7 +487,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.out_sb = a->out_stride_b; sp.out_sh = a->out_stride_h; sp.lse_sb = a->lse_stride_b;
     sp.batch = a->batch; sp.hq = a->num_q_heads; sp.hkv = a->num_kv_heads;
     sp.group = a->num_q_heads / a->num_kv_heads;
-    sp.head_dim = a->head_dim;
+    sp.head_dim = a->head_dim; sp.v_head_dim = v_dim(a);
     sp.page_size = a->page_size; sp.page_shift = ilog2_exact(a->page_size);
     sp.num_splits = S; sp.chunk = r->plan.chunk_tokens; sp.chunk_floor = r->plan.chunk_floor;
     sp.max_tokens = (int32_t)((int64_t)a->max_pages * a->page_size);
@@ -500,7 +519,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.timeline_len = ms && ms->timeline ? ms->timeline_len : 0;
     sp.timeline_rotate = ms ? ms->rotate_heads & 1023 : 0;
     sp.probe = ms && ms->probe_loads ? 1 : 0;
-    if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128))
+    if (sp.probe && (r->plan.algo != FDK_ALGO_MFMA || a->head_dim != 128 || v_dim(a) != 128))
         return fail(FDK_EUNSUPPORTED, "measure: probe_loads is built for the matrix-core path and head_dim 128");
     sp.scale_log2 = a->sm_scale * fdk::kLog2e;
     sp.soft_cap = a->soft_cap > 0.f ? a->soft_cap : 0.f;
@@ -511,7 +530,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     cp.part_o = part_o; cp.part_lse = part_lse; cp.slot_desc = slot_desc; cp.kv_lens = a->kv_lens;
     cp.out = a->out; cp.lse = a->lse;
     cp.out_sb = a->out_stride_b; cp.out_sh = a->out_stride_h; cp.lse_sb = a->lse_stride_b;
-    cp.batch = a->batch; cp.hq = a->num_q_heads; cp.head_dim = a->head_dim;
+    cp.batch = a->batch; cp.hq = a->num_q_heads; cp.head_dim = v_dim(a);
     cp.num_splits = S; cp.chunk = r->plan.chunk_tokens; cp.chunk_floor = r->plan.chunk_floor;
     cp.max_tokens = sp.max_tokens;
     cp.out_dtype = a->out_dtype; cp.pack_lse = sp.pack_lse;
@@ -554,7 +573,7 @@ int decode_impl(const fdk_decode_args* args, void* hip_stream) {
                         (long long)fdk_counters_len(args));
         r.sp.counters = args->counters;
         // the merging workgroup addresses the partials with 32-bit offsets
-        const size_t ws_need = fdk_workspace_bytes(args->batch, args->num_q_heads, args->head_dim, r.plan.num_splits);
+        const size_t ws_need = fdk_workspace_bytes(args->batch, args->num_q_heads, v_dim(args), r.plan.num_splits);
         if ((args->flags & FDK_FLAG_SINGLE_LAUNCH) && ws_need < ((size_t)1 << 32)) {
             r.sp.fused = 1;
             r.sp.ws_bytes = (uint32_t)ws_need;
@@ -644,7 +663,7 @@ int fdk_decode_static(const fdk_decode_args* caller_args, void* hip_stream) {
     a.counters = nullptr;          // one workgroup per item: nothing in the scratch has to start at zero
     a.counters_len = 0;
     if (plan.num_splits > 1) {
-        const size_t need = fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits);
+        const size_t need = fdk_workspace_bytes(a.batch, a.num_q_heads, v_dim(&a), plan.num_splits);
         if (need > kStaticScratchBytes)
             return fail(FDK_EWORKSPACE,
                         "fdk_decode_static: the partials of %d splits need %zu bytes, the static scratch holds %zu; "
@@ -703,8 +722,8 @@ int fdk_combine_ranks(const fdk_combine_ranks_args* caller_args, void* hip_strea
     const fdk_combine_ranks_args* a = &local;
     if (a->num_ranks <= 0 || a->batch < 0 || a->num_q_heads <= 0)
         return fail(FDK_ESHAPE, "bad dims R=%d B=%d Hq=%d", a->num_ranks, a->batch, a->num_q_heads);
-    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
-        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (64, 128 or 256)", a->head_dim);
+    if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 192 && a->head_dim != 256 && a->head_dim != 512)
+        return fail(FDK_EUNSUPPORTED, "head_dim %d not built (values of an output row: 64, 128, 192, 256 or 512)", a->head_dim);
     const bool packed = (a->flags & FDK_FLAG_PACK_LSE) != 0;
     if (elem_size(a->partial_dtype) < 2) return fail(FDK_EUNSUPPORTED, "partial_dtype %d", a->partial_dtype);
     if (elem_size(a->out_dtype) < 2) return fail(FDK_EUNSUPPORTED, "out_dtype %d", a->out_dtype);

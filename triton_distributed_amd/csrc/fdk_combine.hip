@@ -23,7 +23,7 @@ __device__ __forceinline__ float bcast_lane(float x, int i) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), i));
 }
 
-// EPL adjacent fp32 values (EPL in {1, 2, 4}) with one load
+// EPL adjacent fp32 values (EPL = values of an output row / 64) with as few loads as their alignment allows
 template <int EPL> struct Vec;
 template <> struct Vec<1> {
     static __device__ __forceinline__ void load(const float* p, float (&o)[1]) { o[0] = *p; }
@@ -38,6 +38,15 @@ template <> struct Vec<4> {
     static __device__ __forceinline__ void load(const float* p, float (&o)[4]) {
         const float4 v = *reinterpret_cast<const float4*>(p);
         o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec<3> {                       // rows of 192 values: 12 bytes per lane
+    static __device__ __forceinline__ void load(const float* p, float (&o)[3]) { o[0] = p[0]; o[1] = p[1]; o[2] = p[2]; }
+};
+template <> struct Vec<8> {                       // rows of 512 values
+    static __device__ __forceinline__ void load(const float* p, float (&o)[8]) {
+        const float4 v = *reinterpret_cast<const float4*>(p), w = *reinterpret_cast<const float4*>(p + 4);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; o[4] = w.x; o[5] = w.y; o[6] = w.z; o[7] = w.w;
     }
 };
 
@@ -372,13 +381,17 @@ int launch_combine(const CombineParams& p, hipStream_t stream) {
         const int units = p.hg_blocks * p.head_tiles;
         const dim3 grid((unsigned)(p.batch * units));
         const int lpr = p.head_dim / 4;
-        const dim3 block((unsigned)(p.rows_per_slot * lpr > 1024 ? 1024 : p.rows_per_slot * lpr < 64 ? 64 : p.rows_per_slot * lpr));
+        // whole rows only: a row's threads must not start over on another row (48 threads per row of 192 values)
+        const int rows_per_pass = p.rows_per_slot * lpr > 1024 ? 1024 / lpr : p.rows_per_slot;
+        const dim3 block((unsigned)(rows_per_pass * lpr < 64 ? 64 : rows_per_pass * lpr));
         CombineParams q = p;
-        q.rows_per_pass = (int32_t)block.x / lpr;
+        q.rows_per_pass = rows_per_pass;
         switch (p.head_dim) {
             case 64: hipLaunchKernelGGL(combine_slots_kernel<64>, grid, block, 0, stream, q); break;
             case 128: hipLaunchKernelGGL(combine_slots_kernel<128>, grid, block, 0, stream, q); break;
             case 256: hipLaunchKernelGGL(combine_slots_kernel<256>, grid, block, 0, stream, q); break;
+            case 192: hipLaunchKernelGGL(combine_slots_kernel<192>, grid, block, 0, stream, q); break;
+            case 512: hipLaunchKernelGGL(combine_slots_kernel<512>, grid, block, 0, stream, q); break;
             default: return (int)hipErrorInvalidValue;
         }
         return (int)hipGetLastError();
@@ -394,6 +407,8 @@ int launch_combine(const CombineParams& p, hipStream_t stream) {
         case 64: FDK_COMBINE_LAUNCH(64); break;
         case 128: FDK_COMBINE_LAUNCH(128); break;
         case 256: FDK_COMBINE_LAUNCH(256); break;
+        case 192: FDK_COMBINE_LAUNCH(192); break;
+        case 512: FDK_COMBINE_LAUNCH(512); break;
         default: return (int)hipErrorInvalidValue;
     }
 #undef FDK_COMBINE_LAUNCH
@@ -408,6 +423,8 @@ int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream) {
         case 64: hipLaunchKernelGGL(combine_ranks_kernel<64>, grid, dim3(256), 0, stream, p); break;
         case 128: hipLaunchKernelGGL(combine_ranks_kernel<128>, grid, dim3(256), 0, stream, p); break;
         case 256: hipLaunchKernelGGL(combine_ranks_kernel<256>, grid, dim3(256), 0, stream, p); break;
+        case 192: hipLaunchKernelGGL(combine_ranks_kernel<192>, grid, dim3(256), 0, stream, p); break;
+        case 512: hipLaunchKernelGGL(combine_ranks_kernel<512>, grid, dim3(256), 0, stream, p); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();

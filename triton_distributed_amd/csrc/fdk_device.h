@@ -8,7 +8,7 @@
 
 namespace fdk {
 
-constexpr int kHeadDim = 128;       // head dimension of the vector path (the matrix-core path: 64, 128, 256)
+constexpr int kHeadDim = 128;       // head dimension of the vector path (the matrix-core path: see mfma_supported)
 constexpr int kWaveSize = 64;
 constexpr int kBalanceGranule = 16;  // tokens per unit of the balanced partition: one 16-token tile (with 64 tokens a share of a
                                      // few hundred tokens was up to an eighth longer than its neighbours)
@@ -37,6 +37,7 @@ struct SplitParams {
     int64_t tbl_sb;
     int64_t out_sb, out_sh, lse_sb;
     int32_t batch, hq, hkv, group, head_dim;
+    int32_t v_head_dim;             // values per V / output row (head_dim: per q / K row)
     int32_t page_size, page_shift;  // page_shift = log2(page_size) or -1
     int32_t num_splits, chunk;
     int32_t chunk_floor;            // chunk mode, > 0: chunks follow each sequence's own length (chunk_tokens_of)
@@ -80,7 +81,7 @@ struct CombineParams {
     void* out;
     float* lse;
     int64_t out_sb, out_sh, lse_sb;
-    int32_t batch, hq, head_dim;
+    int32_t batch, hq, head_dim;    // head_dim: values per output row
     int32_t num_splits, chunk;
     int32_t chunk_floor;            // as in SplitParams
     int32_t max_tokens;
@@ -142,10 +143,10 @@ int launch_combine_ranks(const CombineRanksParams& p, hipStream_t stream);
 bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);
 // workgroups per (sequence, split) of the VALU path for this head layout
 int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
-bool mfma_supported(int q_dtype, int kv_dtype, int group, int head_dim);
+bool mfma_supported(int q_dtype, int kv_dtype, int group, int head_dim, int v_head_dim);
 int valu_heads_per_wg(int group);
 int mfma_heads_per_wg(int group);
-int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus);
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values);   // row_values: head_dim + v_head_dim
 int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg);
 
 #if defined(__HIPCC__)

@@ -11,6 +11,9 @@ namespace fdk {
 FDK_DECLARE_MFMA(64)
 FDK_DECLARE_MFMA(128)
 FDK_DECLARE_MFMA(256)
+FDK_DECLARE_MFMA(192)            // rows of two segments (128 + 64)
+FDK_DECLARE_MFMA(192v128)        // ... with V rows of 128 values
+FDK_DECLARE_MFMA(576v512)        // 512 + 64, V rows of 512
 #undef FDK_DECLARE_MFMA
 // (the same rule as mfma_work_mode in the kernel header, which this file does not include)
 static int work_mode_of(const SplitParams& p) {
@@ -20,10 +23,15 @@ static int work_mode_of(const SplitParams& p) {
     return p.balanced ? 2 : (p.counters != nullptr && !p.direct && items > resident) ? 1 : 0;
 }
 
-bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim) {
-    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
+// head_dim (q and K rows) / v_head_dim (V and output rows): 64, 128, 256 with V rows alike, 16-bit and fp8 caches;
+// 192 / 192, 192 / 128 and 576 / 512 - rows of two power-of-two segments, as the reference's BLOCK_HEAD_DIM + BLOCK_DPE
+// (flash_decode.py:103-109) - with 16-bit caches
+bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim, int v_head_dim) {
     if (q_dtype != FDK_BF16 && q_dtype != FDK_FP16) return false;
-    return kv_dtype == q_dtype || kv_dtype == FDK_FP8_E4M3;
+    if (head_dim == v_head_dim && (head_dim == 64 || head_dim == 128 || head_dim == 256))
+        return kv_dtype == q_dtype || kv_dtype == FDK_FP8_E4M3;
+    const bool two_segments = (head_dim == 192 && (v_head_dim == 192 || v_head_dim == 128)) || (head_dim == 576 && v_head_dim == 512);
+    return two_segments && kv_dtype == q_dtype;
 }
 
 int mfma_heads_per_wg(int /*group*/) { return 16; }
@@ -37,9 +45,11 @@ int mfma_heads_per_wg(int /*group*/) { return 16; }
 // runs on alone at the end (measured on MI355X: 386 us -> 364 us for B128, 8 kv heads, fp8 cache).
 // Otherwise (the KV range has to be split) two heads per workgroup are the best trade between contiguity and
 // the number of independent workgroups.
-int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus) {
+// (Rows of more than 512 values per token and kv head, K and V together: at most two heads, i.e. the four wavefronts
+// that the registers and the LDS of a compute unit hold at that size.)
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values) {
     const int head_tiles = (group + 15) / 16;
-    for (int nh = 8; nh >= 1; nh >>= 1) {
+    for (int nh = row_values > 512 ? 2 : 8; nh >= 1; nh >>= 1) {
         if (hkv % nh) continue;
         if ((int64_t)batch * (hkv / nh) * head_tiles >= num_cus) return nh;
     }
@@ -54,15 +64,23 @@ int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStre
     if (p.probe) return launch_splitkv_mfma_probe(p, kv_dtype, stream);
     // the ways of handing out pieces are kernels of their own, instantiated in translation units of their own
     const int mode = work_mode_of(p);
-#define FDK_MFMA_CASE(D)                                                                        \
-    case D:                                                                                     \
+#define FDK_MFMA_CASE(D, KEY)                                                                   \
+    case KEY:                                                                                   \
         return mode == 2 ? launch_splitkv_mfma_d##D##_bal(p, q_dtype, kv_dtype, stream)         \
              : mode == 1 ? launch_splitkv_mfma_d##D##_queue(p, q_dtype, kv_dtype, stream)       \
                          : launch_splitkv_mfma_d##D(p, q_dtype, kv_dtype, stream);
+    if (p.v_head_dim != p.head_dim) {
+        switch (p.head_dim * 1024 + p.v_head_dim) {
+            FDK_MFMA_CASE(192v128, 192 * 1024 + 128)
+            FDK_MFMA_CASE(576v512, 576 * 1024 + 512)
+            default: return (int)hipErrorInvalidValue;
+        }
+    }
     switch (p.head_dim) {
-        FDK_MFMA_CASE(64)
-        FDK_MFMA_CASE(128)
-        FDK_MFMA_CASE(256)
+        FDK_MFMA_CASE(64, 64)
+        FDK_MFMA_CASE(128, 128)
+        FDK_MFMA_CASE(256, 256)
+        FDK_MFMA_CASE(192, 192)
         default: return (int)hipErrorInvalidValue;
     }
 #undef FDK_MFMA_CASE

@@ -1,0 +1,10 @@
+// Matrix-core split-KV kernels for q / K rows of 192 values and V rows of 128: one piece per workgroup (single pass, per-sequence chunks).
+#include "fdk_splitkv_mfma.h"
+
+namespace fdk {
+
+int launch_splitkv_mfma_d192v128(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    return launch_mfma_rows2<192, 128, WM_ONE>(p, q_dtype, kv_dtype, stream);
+}
+
+}  // namespace fdk

@@ -138,8 +138,7 @@ def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv
     # the reference's shape asserts, flash_decode.py:851,860
     assert page_size == v_cache.shape[1] and kv_heads == v_cache.shape[2] and k_head_dim == q_head_dim
     assert q_heads % kv_heads == 0
-    if v_cache.shape[-1] != q_head_dim:
-        raise ValueError(f"v head_dim {v_cache.shape[-1]} != q head_dim {q_head_dim} is not built")
+    v_head_dim = v_cache.shape[-1]       # (the reference: V_DIM next to K_DIM, flash_decode.py:103-109; the library says what is built)
     if k_cache.dtype != v_cache.dtype:
         raise ValueError("k_cache and v_cache must share a dtype")
     if q.stride(-1) != 1 or k_cache.stride(-1) != 1 or v_cache.stride(-1) != 1:
@@ -179,6 +178,7 @@ def _fill_args(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv
     a.table_stride_b = block_table.stride(0) if batch > 1 else max(block_table.stride(0), block_table.shape[1])
     a.kv_lens = kv_lens.data_ptr()
     a.batch, a.num_q_heads, a.num_kv_heads, a.head_dim = batch, q_heads, kv_heads, q_head_dim
+    a.v_head_dim = v_head_dim if v_head_dim != q_head_dim else 0
     a.page_size = page_size
     a.max_pages = block_table.shape[1]
     a.max_kv_len = int(max_kv_len) if max_kv_len else 0
@@ -234,7 +234,7 @@ def _args_and_plan(q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap
 def _plan_of(a: FdkDecodeArgs, num_cus: int = 0) -> SplitKvPlan:
     plan = FdkPlan()
     _lib.check(_LIB.fdk_plan(C.byref(a), num_cus, C.byref(plan)))
-    ws = _LIB.fdk_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, plan.num_splits)
+    ws = _LIB.fdk_workspace_bytes(a.batch, a.num_q_heads, a.v_head_dim or a.head_dim, plan.num_splits)
     return SplitKvPlan(plan.num_splits, plan.chunk_tokens, _ALGO_NAMES[plan.algo], int(ws), plan.kv_heads_per_wg,
                        bool(plan.balanced), plan.workgroups, plan.chunk_floor)
 
@@ -408,7 +408,8 @@ def prepare_decode(q, k_cache, v_cache, block_table, kv_lens, sm_scale, *, soft_
     a, plan = _planned if _planned is not None else _args_and_plan(
         q, k_cache, v_cache, block_table, kv_lens, sm_scale, soft_cap, kv_split, max_kv_len, k_scale, v_scale, algo,
         min_kv_len)
-    batch, q_heads, d = q.shape
+    batch, q_heads = q.shape[:2]
+    d = v_cache.shape[-1]                     # values of an output row: V's head dim (the reference's V_DIM)
     measure = None
     if wavefronts or buffers or shares_per_cu or probe_loads or rotate_heads or force_balanced or timeline is not None:
         measure = FdkMeasureArgs()
@@ -573,7 +574,8 @@ def gqa_fwd_batch_decode_intra_rank(q, k_cache, v_cache, workspace, q_lens, kv_l
     ``length_feedback`` (not in the reference): a ``LengthFeedback`` that the caller keeps for this batch; the call
     plans with the bounds the previous call left there and leaves its own (see ``LengthFeedback``).  Without it the
     call knows nothing about the lengths and every call plans alike."""
-    batch, q_heads, d = q.shape
+    batch, q_heads = q.shape[:2]
+    d = v_cache.shape[-1]
     if output_combine is None:
         output_combine = torch.empty((batch, q_heads, d + 1), dtype=q.dtype, device=q.device)
     if q.is_cuda:

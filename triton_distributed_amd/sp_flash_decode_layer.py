@@ -27,8 +27,8 @@ class SpGQAFlashDecodeAttention(torch.nn.Module):
                  scale=1, soft_cap=0, max_allowed_batch=1, thrink_buffer_threshold=500, stages=20,
                  all_gather: Optional[Callable[[torch.Tensor], torch.Tensor]] = None, length_feedback: bool = True):
         super().__init__()
-        if q_head_dim != v_head_dim:
-            raise ValueError("q_head_dim != v_head_dim is not built")
+        # (which pairs are built - 64, 128, 256 alike; 192 with 192 or 128; 576 with 512 - is for the library to say, at the
+        # first decode)
         if num_ranks > 1 and all_gather is None:
             raise ValueError("num_ranks > 1 needs an all_gather callable: this package contains no collective")
         self.rank, self.node, self.num_ranks, self.num_nodes = rank, node, num_ranks, num_nodes

@@ -32,6 +32,11 @@ class DecodeConfig:
     q_dtype: str = "bf16"                # "bf16" | "fp16"
     spare_pages: int = 64
     description: str = ""
+    v_head_dim: int = 0                  # values per V / output row where they differ from head_dim (q and K rows)
+
+    @property
+    def dv(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 CONFIGS: Dict[str, DecodeConfig] = {
@@ -54,6 +59,16 @@ CONFIGS["ragged_b64_8kv"] = DecodeConfig("ragged_b64_8kv", 1201, 64, 32, 8, 128,
                                          description="B64 32q/8kv D128 N~U[1,8192] P16 bf16")
 CONFIGS["fp8_8b_b32"] = DecodeConfig("fp8_8b_b32", 1202, 32, 32, 8, 128, 16, kv_len=4096, kv_dtype="fp8_e4m3",
                                      description="B32 32q/8kv D128 N4096 P16, e4m3 KV with per-kv-head scales")
+
+# q / K rows of two segments and V rows of their own length (the reference's BLOCK_HEAD_DIM + BLOCK_DPE and V_DIM,
+# flash_decode.py:103-109): the headline shape with 192-value rows, with V rows of 128, and a latent-attention decode
+# shape (one shared kv head of 512 + 64 values, 128 q heads, V = 512 values).
+CONFIGS["d192_b32"] = DecodeConfig("d192_b32", 1301, 32, 32, 8, 192, 16, kv_len=4096,
+                                   description="B32 32q/8kv Dk192 Dv192 N4096 P16 bf16")
+CONFIGS["d192v128_b32"] = DecodeConfig("d192v128_b32", 1302, 32, 32, 8, 192, 16, kv_len=4096, v_head_dim=128,
+                                       description="B32 32q/8kv Dk192 Dv128 N4096 P16 bf16")
+CONFIGS["d576v512_b32"] = DecodeConfig("d576v512_b32", 1303, 32, 128, 1, 576, 64, kv_len=4096, v_head_dim=512,
+                                       description="B32 128q/1kv Dk576 Dv512 N4096 P64 bf16")
 
 # The shape behind the reference's only published figure for this path (README.md:200-202; perf loops of
 # test/nvidia/test_sp_decode_attn.py:203-220 and test_decode_attn.py:294-527): batch 1, 96 q / 12 kv heads,
@@ -92,8 +107,8 @@ class DecodeInputs:
         e_kv = 1 if c.kv_dtype == "fp8_e4m3" else 2
         tokens = sum(self.kv_lens_host)
         pages = sum((n + c.page_size - 1) // c.page_size for n in self.kv_lens_host)
-        total = tokens * c.kv_heads * 2 * c.head_dim * e_kv
-        total += 2 * c.batch * c.q_heads * c.head_dim * 2        # q + out
+        total = tokens * c.kv_heads * (c.head_dim + c.dv) * e_kv
+        total += c.batch * c.q_heads * (c.head_dim + c.dv) * 2   # q + out
         total += c.batch * c.q_heads * 4                          # lse
         total += 4 * pages + 4 * c.batch
         if c.kv_dtype == "fp8_e4m3":
@@ -102,7 +117,7 @@ class DecodeInputs:
 
     def flops(self) -> int:
         c = self.cfg
-        return 4 * c.q_heads * c.head_dim * sum(self.kv_lens_host)
+        return 2 * c.q_heads * (c.head_dim + c.dv) * sum(self.kv_lens_host)
 
 
 def quantize_kv_fp8(cache: torch.Tensor, chunk_pages: int = 4096):
@@ -163,7 +178,7 @@ def make_inputs(name_or_cfg, device="cpu", poison_tail: bool = False) -> DecodeI
         q = (q.float() * cfg.q_scale).to(dt)
     cache_shape = (pool, cfg.page_size, cfg.kv_heads, cfg.head_dim)
     k_cache = _randn_bf16(cache_shape, gen, dtype=dt)
-    v_cache = _randn_bf16(cache_shape, gen, dtype=dt)
+    v_cache = _randn_bf16(cache_shape[:3] + (cfg.dv,), gen, dtype=dt)
     k_scale = v_scale = None
     if cfg.kv_dtype == "fp8_e4m3":
         k_cache, k_scale = quantize_kv_fp8(k_cache)
@@ -179,4 +194,4 @@ def scaled_down(cfg: DecodeConfig, batch: Optional[int] = None, kv_len: Optional
     return DecodeConfig(cfg.name + "_small", cfg.seed, batch or cfg.batch, cfg.q_heads, cfg.kv_heads, cfg.head_dim,
                         cfg.page_size, kv_len if cfg.kv_len is not None else None,
                         kv_len_range if cfg.kv_len is None else None, cfg.q_scale, cfg.kv_dtype, cfg.q_dtype,
-                        min(cfg.spare_pages, 8), cfg.description)
+                        min(cfg.spare_pages, 8), cfg.description, cfg.v_head_dim)
