@@ -280,7 +280,7 @@ def test_two_segment_head_dims_in_every_plan(cuda_device, dims, page):
     g = torch.Generator().manual_seed(dk + dv + page)
     lens = [int(x) for x in torch.randint(1, 3000, (12,), generator=g)]
     lens[3], lens[7] = 0, 1
-    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, (16, 2), page, torch.bfloat16, 77 + page, table_extra=2)
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, (48, 2), page, torch.bfloat16, 77 + page, table_extra=2)   # two q-head tiles per kv head, the second half full
     ref_plan = tda.get_split_kv_plan(q, k, v, table, lens_t, scale)
     assert ref_plan.algo == "mfma"
     live = [i for i, n in enumerate(lens) if n > 0]
@@ -294,7 +294,7 @@ def test_two_segment_head_dims_in_every_plan(cuda_device, dims, page):
     assert plan_b.balanced
     out_c, lse_c = tda.flash_decode(q, k, v, table, lens_t, scale, kv_split=5)
     out_q, lse_q = tda.flash_decode(q, k, v, table, lens_t, scale, kv_split=48)      # 12 x 48 pieces: more than are resident, a queue
-    out_f = torch.empty(len(lens), 16, dv, dtype=torch.float32, device=cuda_device)
+    out_f = torch.empty(len(lens), 48, dv, dtype=torch.float32, device=cuda_device)
     _, lse_f = tda.flash_decode(q, k, v, table, lens_t, scale, out=out_f)
     torch.cuda.synchronize()
     check(out_b, lse_b, "equal shares")
@@ -326,7 +326,7 @@ def test_two_segment_head_dims_random_shapes(cuda_device, seed):
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
     dims = TWO_SEGMENT_DIMS[seed % 3]
     hkv = [1, 2, 3, 4, 8][r(0, 4)]
-    group = [1, 2, 4, 7, 8, 16, 20][r(0, 6)]
+    group = [1, 2, 4, 7, 8, 16, 20, 40][r(0, 7)]
     page = [1, 2, 5, 8, 16, 32, 48, 128][r(0, 7)]
     batch = r(1, 20)
     top = [60, 700, 5000][r(0, 2)]

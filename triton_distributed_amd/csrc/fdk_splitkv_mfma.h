@@ -258,17 +258,38 @@ __device__ __forceinline__ void merge_rows(const SplitParams& p, const int64_t (
 enum WorkMode { WM_ONE = 0,     // one piece per workgroup: single pass, per-sequence chunks
                 WM_QUEUE = 1,   // chunk mode, a fixed set of workgroups pulls the pieces from a queue
                 WM_SHARES = 2 };// balanced mode: equal shares of the whole batch
+// Several q-head tiles per kv head (groups of more than 16 heads) read the same K / V rows.  Workgroups go to the eight
+// XCDs round-robin in linear order and every XCD has an L2 of its own: with the tile index running fastest, the tiles of
+// a row of work (a kv-head block of a sequence's piece) land on different XCDs and each of them fetches the rows from
+// memory.  This maps the linear workgroup id so that the T tiles of a row sit on ONE XCD, within 8 T consecutive ids
+// (they run at the same time and share what the first of them brought into the L2):
+// id = block * 8 T + tile * 8 + slot  ->  row = block * 8 + slot.  Rows past the last full block of eight keep the plain order.
+__device__ __forceinline__ void tiles_on_one_xcd(int id, int rows, int T, int& row, int& tile) {
+    const int full_rows = rows & ~7;
+    if (id < full_rows * T) {
+        const int blk = id / (8 * T), in = id - blk * 8 * T;
+        tile = in >> 3;
+        row = blk * 8 + (in & 7);
+    } else {
+        const int rest = id - full_rows * T;
+        row = full_rows + rest / T;
+        tile = rest % T;
+    }
+}
+
 // head_dim 64, 128, 256 (K and V rows alike, one segment)
 template <int QDT, bool FP8, int PM, int NBUF, int D, bool PROBE = false, int MODE = WM_ONE>
 __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) {
     constexpr int DK = D, DV = D;
+    constexpr bool REUSE = false;
 #include "fdk_splitkv_mfma_body.h"
 }
 // Rows of two segments and V rows shorter than K rows (q / K rows of DK values, V / output rows of DV): 16-bit caches,
 // one register buffer.  Beyond 512 values per token and kv head a workgroup has four wavefronts, each alone on its
 // SIMD with the whole register file.
 constexpr int rows2_max_threads(int dk, int dv) { return dk + dv > 512 ? 256 : 512; }
-template <int QDT, int PM, int DK, int DV, int MODE>
+// REUSE: several workgroups read the same K / V rows (more than one q-head tile per kv head).
+template <int QDT, int PM, int DK, int DV, int MODE, bool REUSE>
 __global__ __launch_bounds__(rows2_max_threads(DK, DV)) void splitkv_mfma_rows2_kernel(const SplitParams p) {
     constexpr bool FP8 = false, PROBE = false;
     constexpr int NBUF = 1;
@@ -390,21 +411,25 @@ int launch_rows2(const SplitParams& p_in, hipStream_t stream) {
     p.shares = (int32_t)grid.y;
     p.grid_x = (int32_t)grid.x;
     p.wavefronts = nw;
+    const bool reuse = p.head_tiles > 1;
+#define FDK_ROWS2_LAUNCH(PMV, RU)                                                                                          \
+    do {                                                                                                                   \
+        if (lds_bytes > 64 * 1024) {                                                                                       \
+            const hipError_t e = hipFuncSetAttribute(                                                                      \
+                reinterpret_cast<const void*>(&splitkv_mfma_rows2_kernel<QDT, PMV, DK, DV, MODE, RU>),                     \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);                                               \
+            if (e != hipSuccess) return (int)e;                                                                            \
+        }                                                                                                                  \
+        hipLaunchKernelGGL((splitkv_mfma_rows2_kernel<QDT, PMV, DK, DV, MODE, RU>), grid, block, lds_bytes, stream, p);    \
+    } while (0)
     if (pm == PM_TILE) {
-        if (lds_bytes > 64 * 1024) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&splitkv_mfma_rows2_kernel<QDT, PM_TILE, DK, DV, MODE>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) return (int)e;
-        }
-        hipLaunchKernelGGL((splitkv_mfma_rows2_kernel<QDT, PM_TILE, DK, DV, MODE>), grid, block, lds_bytes, stream, p);
+        if (reuse) FDK_ROWS2_LAUNCH(PM_TILE, true);
+        else FDK_ROWS2_LAUNCH(PM_TILE, false);
     } else {
-        if (lds_bytes > 64 * 1024) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&splitkv_mfma_rows2_kernel<QDT, PM_ROW, DK, DV, MODE>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) return (int)e;
-        }
-        hipLaunchKernelGGL((splitkv_mfma_rows2_kernel<QDT, PM_ROW, DK, DV, MODE>), grid, block, lds_bytes, stream, p);
+        if (reuse) FDK_ROWS2_LAUNCH(PM_ROW, true);
+        else FDK_ROWS2_LAUNCH(PM_ROW, false);
     }
+#undef FDK_ROWS2_LAUNCH
     return (int)hipGetLastError();
 }
 

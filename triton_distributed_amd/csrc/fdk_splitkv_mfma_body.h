@@ -1,5 +1,5 @@
 // The body of the matrix-core split-KV kernels (fdk_splitkv_mfma.h includes this file inside each of its two kernel
-// definitions, which supply: QDT, FP8, PM, NBUF, PROBE, MODE, DK = values per q and K row, DV = values per V and
+// definitions, which supply: QDT, FP8, PM, NBUF, PROBE, MODE, REUSE, DK = values per q and K row, DV = values per V and
 // output row, and the argument block p).  Kept as text shared by the two kernels rather than as a function they
 // call: the kernel arguments then stay where the compiler reads them with scalar loads.
     constexpr bool BAL = MODE == WM_SHARES;
@@ -164,6 +164,10 @@
     const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
     // Rows of two segments: the row of the tile and the byte of the cache row that this lane's 16 bytes of load
     // instruction j start at (j is a constant wherever these are used)
+    // (rows of two segments) K / V rows that several workgroups read - the q-head tiles of one kv head, which share an
+    // XCD, see tiles_on_one_xcd - come by plain loads, so that they stay in that XCD's L2 for the other tiles; rows
+    // that are read once, with the non-temporal hint
+    auto load_rows16 = [&](const void* ptr) { return REUSE ? *reinterpret_cast<const uint4*>(ptr) : load_stream16(ptr); };
     auto k_row = [&](int j) { return RK::row0(j) + lane / RK::lpr(j); };
     auto v_row = [&](int j) { return RV::row0(j) + lane / RV::lpr(j); };
     auto k_byte = [&](int j) { return RK::seg_byte(j) + (lane % RK::lpr(j)) * 16; };
@@ -210,9 +214,9 @@
                 return (uint64_t)pg * sp_bytes + (uint64_t)(slot * st_bytes);
             };
 #pragma unroll
-            for (int j = 0; j < NJK; ++j) put(rg.k[j], load_stream16(kplane + k_byte(j) + row_at(k_row(j), ksp_bytes, kst_bytes)));
+            for (int j = 0; j < NJK; ++j) put(rg.k[j], load_rows16(kplane + k_byte(j) + row_at(k_row(j), ksp_bytes, kst_bytes)));
 #pragma unroll
-            for (int j = 0; j < NJV; ++j) put(rg.v[j], load_stream16(vplane + v_byte(j) + row_at(v_row(j), vsp_bytes, vst_bytes)));
+            for (int j = 0; j < NJV; ++j) put(rg.v[j], load_rows16(vplane + v_byte(j) + row_at(v_row(j), vsp_bytes, vst_bytes)));
         }
     };
 
@@ -256,10 +260,10 @@
             } else {
 #pragma unroll
                 for (int j = 0; j < NJK; ++j)
-                    put(rg.k[j], load_stream16(kp + (int64_t)RK::row0(j) * p.k_st * ES + koff[j < RK::NJ0 ? 0 : 1]));
+                    put(rg.k[j], load_rows16(kp + (int64_t)RK::row0(j) * p.k_st * ES + koff[j < RK::NJ0 ? 0 : 1]));
 #pragma unroll
                 for (int j = 0; j < NJV; ++j)
-                    put(rg.v[j], load_stream16(vp + (int64_t)RV::row0(j) * p.v_st * ES + voff[j < RV::NJ0 ? 0 : 1]));
+                    put(rg.v[j], load_rows16(vp + (int64_t)RV::row0(j) * p.v_st * ES + voff[j < RV::NJ0 ? 0 : 1]));
             }
         } else {
             issue(t, pi, rg, BoolTag<false>());
@@ -615,14 +619,25 @@
             // grid = (head blocks x head tiles, splits, sequences): the piece follows from the block index without a
             // division, so the table and q loads of the piece can be requested as soon as the arguments are there.
             // (Workgroups are handed out in x-major order: neighbours still read neighbouring heads of the same tokens.)
-            const int split = blockIdx.y, pb = blockIdx.z;
+            int split = blockIdx.y, pb = blockIdx.z;
             int ht = 0, hgb = blockIdx.x;
 #ifdef FDK_TIMELINE
             if (p.head_tiles == 1) hgb = (int)((blockIdx.x + (unsigned)p.timeline_rotate) % (unsigned)p.grid_x);
 #endif
-            if (p.head_tiles > 1) {
-                ht = blockIdx.x % p.head_tiles;
-                hgb = blockIdx.x / p.head_tiles;
+            if constexpr (kOneSegment) {
+                if (p.head_tiles > 1) {
+                    ht = blockIdx.x % p.head_tiles;
+                    hgb = blockIdx.x / p.head_tiles;
+                }
+            } else if (p.head_tiles > 1) {
+                // the q-head tiles of a (sequence, split, kv-head block) on one XCD: see tiles_on_one_xcd
+                int row;
+                tiles_on_one_xcd((int)(blockIdx.x + p.grid_x * (blockIdx.y + p.num_splits * blockIdx.z)),
+                                 p.hg_blocks * p.num_splits * p.batch, p.head_tiles, row, ht);
+                hgb = row % p.hg_blocks;
+                row /= p.hg_blocks;
+                split = row % p.num_splits;
+                pb = row / p.num_splits;
             }
             // the last split runs to the end of the sequence: a max_kv_len hint that was too small costs balance, not tokens
             const int64_t unit_row0 = ((int64_t)pb * p.hq + hgb * nh * p.group + ht * 16) * p.num_splits;
@@ -705,7 +720,16 @@
         };
         int x = 0, hi = 0;                            // next granule, end of this workgroup's share
         int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
-        const int wc = blockIdx.y, bu = blockIdx.x;   // grid = (units, shares)
+        int wc_of_wg = blockIdx.y, bu_of_wg = blockIdx.x;   // grid = (units, shares)
+        if constexpr (!kOneSegment) {
+            if (p.head_tiles > 1) {                         // the q-head tiles of a (share, kv-head block) on one XCD
+                int row, tile;
+                tiles_on_one_xcd((int)(blockIdx.x + p.grid_x * blockIdx.y), p.hg_blocks * p.shares, p.head_tiles, row, tile);
+                bu_of_wg = (row % p.hg_blocks) * p.head_tiles + tile;
+                wc_of_wg = row / p.hg_blocks;
+            }
+        }
+        const int wc = wc_of_wg, bu = bu_of_wg;
         int share_q = 1, share_r = 0;                 // granules per share, shares with one more
         // the piece of sequence b in this workgroup's share, and where the share's part of the sequence ends
         auto piece_of = [&](int& piece_end) {
