@@ -353,6 +353,41 @@ def test_two_segment_head_dims_random_shapes(cuda_device, seed):
            ref_tol=4e-2 if scale > dims[0] ** -0.5 else None)
 
 
+@pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
+def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(cuda_device, dims):
+    """A captured call (the kernels of the widest rows ask for more LDS than the default limit at launch) replayed on
+    changed q and lengths, and the entry point that allocates nothing, against the eager call."""
+    dk, dv = dims
+    g = torch.Generator().manual_seed(dk * 3 + dv)
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, [2500] * 4, (32, 2), 16, torch.bfloat16, 31)   # pages for every length below
+    lens_t.copy_(_lens_t([2500, 1, 900, 1800], cuda_device))
+    scale = dk ** -0.5
+    call = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500)
+    assert call.plan.num_splits > 1
+    call.run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call.run()
+    for i, new_lens in enumerate(([2500, 1, 900, 1800], [7, 2400, 0, 333], [1200, 1200, 1200, 1200])):
+        lens_t.copy_(_lens_t(new_lens, cuda_device))
+        q.copy_(torch.randn(q.shape, generator=g).to(torch.bfloat16).to(cuda_device))
+        call.out.fill_(float("nan"))
+        call.lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_o, got_l = call.out.clone(), call.lse.clone()
+        want_o, want_l = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=2500)
+        static = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500, static_scratch=True)
+        st_o, st_l = static.run_static()
+        torch.cuda.synchronize()
+        assert torch.equal(got_o, want_o) and torch.equal(got_l, want_l), f"replay {i}"
+        assert torch.equal(st_o, want_o) and torch.equal(st_l, want_l), f"static entry {i}"
+        live = [j for j, n in enumerate(new_lens) if n > 0]
+        _check(got_o[live], got_l[live], q[live], k, v, table[live], [new_lens[j] for j in live], scale,
+               tag=f"dims={dims} graph replay {i}")
+
+
 def test_what_is_not_built_for_two_segment_head_dims_is_refused(cuda_device):
     q, k, v, table, lens_t = _two_segment_inputs(cuda_device, (192, 128), [300, 20], (8, 2), 16, torch.bfloat16, 5)
     with pytest.raises(ValueError, match="matrix-core"):
