@@ -388,6 +388,46 @@ def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(
                tag=f"dims={dims} graph replay {i}")
 
 
+@pytest.mark.parametrize("heads", [(128, 1), (128, 2), (64, 1), (40, 1), (66, 2)])
+@pytest.mark.parametrize("page", [64, 16, 6, 1])
+def test_large_groups_on_one_kv_head_share_the_staged_tiles(cuda_device, heads, page):
+    """More than 32 q heads per kv head with rows of 576 / 512 values (latent attention): the workgroups cover 64 q heads
+    of a kv head and their wavefronts share every staged tile.  Every way of handing out the pieces, groups that fill
+    the last workgroup or wavefront only partly, empty sequences, fp16, a soft cap."""
+    dims = (576, 512)
+    hq, hkv = heads
+    scale = 576 ** -0.5
+    g = torch.Generator().manual_seed(hq * 7 + hkv + page)
+    lens = [int(x) for x in torch.randint(1, 2200, (7,), generator=g)]
+    lens[2], lens[5] = 0, 1
+    dtype = torch.float16 if page == 16 else torch.bfloat16
+    cap = 25.0 if page == 6 else 0.0
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, heads, page, dtype, 300 + hq + page, table_extra=1)
+    live = [i for i, n in enumerate(lens) if n > 0]
+
+    def check(o, l, tag):
+        assert o.shape == (len(lens), hq, 512)
+        assert torch.isfinite(o.float()).all() and float(o[2].abs().max()) == 0 and bool((l[2] == -math.inf).all()), tag
+        _check(o[live], l[live], q[live], k, v, table[live], [lens[i] for i in live], scale, cap, tag=f"heads={heads} P={page} {tag}")
+
+    plan = tda.get_split_kv_plan(q, k, v, table, lens_t, scale)
+    assert plan.algo == "mfma" and plan.kv_heads_per_wg == 1
+    out_a, lse_a = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap)
+    out_1, lse_1 = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, kv_split=1)
+    out_c, lse_c = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, kv_split=5)
+    out_q, lse_q = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, kv_split=40)       # a work queue
+    out_b, lse_b = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, force_balanced=True)
+    assert tda.get_split_kv_plan(q, k, v, table, lens_t, scale, force_balanced=True).balanced
+    out_h, lse_h = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, max_kv_len=max(lens), min_kv_len=max(lens))
+    packed = tda.gqa_fwd_batch_decode_intra_rank(q, k, v, None, None, lens_t, table, scale, cap, kv_split=32)
+    torch.cuda.synchronize()
+    for o, l, tag in ((out_a, lse_a, "auto"), (out_1, lse_1, "single pass"), (out_c, lse_c, "5 chunks"), (out_q, lse_q, "queue"),
+                      (out_b, lse_b, "equal shares"), (out_h, lse_h, "alike lengths")):
+        check(o, l, tag)
+    torch.testing.assert_close(packed[..., :512].float(), out_a.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(packed[live][..., 512].float(), lse_a[live], atol=3e-2, rtol=1e-2)
+
+
 def test_what_is_not_built_for_two_segment_head_dims_is_refused(cuda_device):
     q, k, v, table, lens_t = _two_segment_inputs(cuda_device, (192, 128), [300, 20], (8, 2), 16, torch.bfloat16, 5)
     with pytest.raises(ValueError, match="matrix-core"):

@@ -35,6 +35,8 @@ SOURCES = [
     "fdk_splitkv_mfma_d192.hip", "fdk_splitkv_mfma_d192_queue.hip", "fdk_splitkv_mfma_d192_bal.hip",
     "fdk_splitkv_mfma_d192v128.hip", "fdk_splitkv_mfma_d192v128_queue.hip", "fdk_splitkv_mfma_d192v128_bal.hip",
     "fdk_splitkv_mfma_d576v512.hip", "fdk_splitkv_mfma_d576v512_queue.hip", "fdk_splitkv_mfma_d576v512_bal.hip",
+    # ... large q-head groups on one kv head: the wavefronts of a workgroup share the staged tiles
+    "fdk_splitkv_mfma_d576v512_shared.hip", "fdk_splitkv_mfma_d576v512_shared_queue.hip", "fdk_splitkv_mfma_d576v512_shared_bal.hip",
 ]
 
 # the translation units that contain the matrix-core split kernel: the only ones the timeline build compiles anew

@@ -284,9 +284,10 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const bool heads_contiguous = a->k_stride_head == a->head_dim && a->v_stride_head == a->head_dim;
     int kv_heads_per_wg = 1;
     int units_per_seq;
+    const int tile_heads = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a)) : 16;   // q heads of a kv head per workgroup
     if (algo == FDK_ALGO_MFMA) {
         kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus, a->head_dim + v_dim(a));
-        units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg);
+        units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg, tile_heads);
     } else {
         units_per_seq = fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
     }
@@ -323,7 +324,8 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         }
         if (rebalance) {
             kv_heads_per_wg = a->num_kv_heads % 2 ? 1 : 2;
-            units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg);
+            if (tile_heads > 16) kv_heads_per_wg = 1;
+            units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg, tile_heads);
         }
     }
 
@@ -392,7 +394,7 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
         // Deriving the partition costs every workgroup a pass over kv_lens before its first load: worth it
         // only when a share is long enough to hide that.
         if (share_tokens >= kMinBalancedShare || force_balanced) {
-            const int64_t rows_per_slot = (int64_t)kv_heads_per_wg * (group < 16 ? group : 16);
+            const int64_t rows_per_slot = (int64_t)kv_heads_per_wg * (group < tile_heads ? group : tile_heads);
             const int64_t rows = (shares + batch) * units_per_seq * rows_per_slot;
             plan->balanced = 1;
             plan->workgroups = (int32_t)(shares * units_per_seq);
@@ -438,7 +440,7 @@ int piece_cost_granules(const fdk_decode_args* a, int kv_heads_per_wg) {
 // q-head tiles per kv head, as the resolved algorithm's kernel counts them
 int head_tiles_of(const fdk_decode_args* a, int algo) {
     const int group = a->num_q_heads / a->num_kv_heads;
-    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group) : fdk::valu_heads_per_wg(group);
+    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a)) : fdk::valu_heads_per_wg(group);
     return (group + hpw - 1) / hpw;
 }
 
@@ -495,7 +497,8 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.hg_per_wg = r->plan.kv_heads_per_wg;
     sp.balanced = r->plan.balanced;
     sp.workgroups = r->plan.workgroups;
-    sp.heads_per_tile = sp.group < 16 ? sp.group : 16;
+    sp.tile_heads = r->plan.algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(sp.group, a->head_dim + v_dim(a)) : 16;
+    sp.heads_per_tile = sp.group < sp.tile_heads ? sp.group : sp.tile_heads;
     sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
     sp.piece_cost = sp.balanced ? piece_cost_granules(a, sp.hg_per_wg) : 0;
     const fdk_measure_args* const ms = a->measure;
@@ -537,7 +540,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     cp.balanced = sp.balanced; cp.workgroups = sp.workgroups;
     cp.group = sp.group; cp.kv_heads_per_wg = sp.hg_per_wg; cp.head_tiles = sp.head_tiles;
     cp.hg_blocks = a->num_kv_heads / (sp.hg_per_wg > 0 ? sp.hg_per_wg : 1);
-    cp.rows_per_slot = sp.rows_per_slot; cp.heads_per_tile = sp.heads_per_tile;
+    cp.rows_per_slot = sp.rows_per_slot; cp.heads_per_tile = sp.heads_per_tile; cp.tile_heads = sp.tile_heads;
     cp.piece_cost = sp.piece_cost;
     cp.length_feedback = a->length_feedback;
     cp.feedback_epoch = this_epoch;

@@ -258,13 +258,13 @@ __global__ __launch_bounds__(1024) void combine_slots_kernel(const CombineParams
     const int2 desc = p.slot_desc[blockIdx.x];                  // (garbage for a sequence without tokens: not used)
     const int kv_len = p.kv_lens[b];
     const int hgb = u / p.head_tiles, ht = u % p.head_tiles;
-    const int heads_here = min(16, p.group - ht * 16);
+    const int heads_here = min(p.tile_heads, p.group - ht * p.tile_heads);
     const int c4 = threadIdx.x % LPR;
     const int64_t piece_step = (int64_t)units * p.rows_per_slot;                 // rows from one piece to the next
     for (int r = threadIdx.x / LPR; r < p.rows_per_slot; r += p.rows_per_pass) {
         const int hl = r / p.heads_per_tile, g = r % p.heads_per_tile;
         if (g >= heads_here) continue;                                       // the last tile of a group may be short
-        const int hq = (hgb * p.kv_heads_per_wg + hl) * p.group + ht * 16 + g;
+        const int hq = (hgb * p.kv_heads_per_wg + hl) * p.group + ht * p.tile_heads + g;
         const int64_t ob = (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         float inv = 0.f, lse = -INFINITY;                                    // no tokens: out = 0, lse = -inf

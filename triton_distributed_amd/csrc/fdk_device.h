@@ -55,7 +55,9 @@ struct SplitParams {
     int32_t shares;                 // balanced mode: gridDim.y
     int32_t grid_x;                 // gridDim.x
     int32_t wavefronts;             // blockDim.x / 64
-    int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= 16)
+    int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= tile_heads)
+    int32_t tile_heads;             // q heads of a kv head that one workgroup covers: 16 (an MFMA tile), or 64 in the
+                                    // kernels whose wavefronts share the staged tiles (fdk_splitkv_mfma_shared.h)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
     int32_t* length_feedback;       // set where this kernel ends the call: {min, max of the clamped kv_lens, epoch, batch} goes here
@@ -91,6 +93,7 @@ struct CombineParams {
     int32_t balanced, workgroups;
     int32_t group, kv_heads_per_wg, head_tiles, hg_blocks, rows_per_slot, heads_per_tile, piece_cost;
     int32_t rows_per_pass;          // balanced mode: rows of a slot the workgroup covers at once (blockDim.x / (head_dim / 4))
+    int32_t tile_heads;             // as in SplitParams
     int32_t* length_feedback;       // as in SplitParams (null: nothing is stored)
     int32_t feedback_epoch;
 };
@@ -145,9 +148,9 @@ bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);
 int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
 bool mfma_supported(int q_dtype, int kv_dtype, int group, int head_dim, int v_head_dim);
 int valu_heads_per_wg(int group);
-int mfma_heads_per_wg(int group);
+int mfma_heads_per_wg(int group, int row_values);   // q heads of a kv head per workgroup (SplitParams.tile_heads)
 int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values);   // row_values: head_dim + v_head_dim
-int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg);
+int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg, int tile_heads);
 
 #if defined(__HIPCC__)
 

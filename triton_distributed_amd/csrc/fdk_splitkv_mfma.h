@@ -283,6 +283,7 @@ __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) 
     constexpr int DK = D, DV = D;
     constexpr bool REUSE = false;
 #include "fdk_splitkv_mfma_body.h"
+#include "fdk_splitkv_mfma_work.h"
 }
 // Rows of two segments and V rows shorter than K rows (q / K rows of DK values, V / output rows of DV): 16-bit caches,
 // one register buffer.  Beyond 512 values per token and kv head a workgroup has four wavefronts, each alone on its
@@ -294,6 +295,7 @@ __global__ __launch_bounds__(rows2_max_threads(DK, DV)) void splitkv_mfma_rows2_
     constexpr bool FP8 = false, PROBE = false;
     constexpr int NBUF = 1;
 #include "fdk_splitkv_mfma_body.h"
+#include "fdk_splitkv_mfma_work.h"
 }
 
 // Whether the call runs as a work queue: whenever the KV range is split into per-sequence chunks, the caller provided

@@ -14,6 +14,7 @@ FDK_DECLARE_MFMA(256)
 FDK_DECLARE_MFMA(192)            // rows of two segments (128 + 64)
 FDK_DECLARE_MFMA(192v128)        // ... with V rows of 128 values
 FDK_DECLARE_MFMA(576v512)        // 512 + 64, V rows of 512
+FDK_DECLARE_MFMA(576v512_shared) // ... large q-head groups: wavefronts share the staged tiles
 #undef FDK_DECLARE_MFMA
 // (the same rule as mfma_work_mode in the kernel header, which this file does not include)
 static int work_mode_of(const SplitParams& p) {
@@ -34,7 +35,10 @@ bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim, int 
     return two_segments && kv_dtype == q_dtype;
 }
 
-int mfma_heads_per_wg(int /*group*/) { return 16; }
+// q heads of one kv head that a workgroup covers: a tile of 16 (a wavefront per kv head), or 64 where the rows are
+// long and the group is large - latent attention, 128 q heads on one kv head of 576 + 512 values - and the kernels of
+// fdk_splitkv_mfma_shared.h load and stage every tile once for four tiles of 16 q heads
+int mfma_heads_per_wg(int group, int row_values) { return row_values > 512 && group > 32 ? 64 : 16; }
 
 // kv heads per workgroup.  Adjacent kv heads of a token are adjacent in the cache, so a workgroup that takes
 // several heads reads longer contiguous runs per token.  When the (sequence, head block) units alone fill the
@@ -48,6 +52,7 @@ int mfma_heads_per_wg(int /*group*/) { return 16; }
 // (Rows of more than 512 values per token and kv head, K and V together: at most two heads, i.e. the four wavefronts
 // that the registers and the LDS of a compute unit hold at that size.)
 int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values) {
+    if (mfma_heads_per_wg(group, row_values) > 16) return 1;          // the shared-tile kernels: one kv head, 64 q heads
     const int head_tiles = (group + 15) / 16;
     for (int nh = row_values > 512 ? 2 : 8; nh >= 1; nh >>= 1) {
         if (hkv % nh) continue;
@@ -56,8 +61,8 @@ int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_val
     return hkv % 2 ? 1 : 2;
 }
 
-int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg) {
-    return (hkv / kv_heads_per_wg) * ((group + 15) / 16);
+int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg, int tile_heads) {
+    return (hkv / kv_heads_per_wg) * ((group + tile_heads - 1) / tile_heads);
 }
 
 int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
@@ -69,6 +74,12 @@ int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStre
         return mode == 2 ? launch_splitkv_mfma_d##D##_bal(p, q_dtype, kv_dtype, stream)         \
              : mode == 1 ? launch_splitkv_mfma_d##D##_queue(p, q_dtype, kv_dtype, stream)       \
                          : launch_splitkv_mfma_d##D(p, q_dtype, kv_dtype, stream);
+    if (p.tile_heads > 16) {
+        switch (p.head_dim * 1024 + p.v_head_dim) {
+            FDK_MFMA_CASE(576v512_shared, 576 * 1024 + 512)
+            default: return (int)hipErrorInvalidValue;
+        }
+    }
     if (p.v_head_dim != p.head_dim) {
         switch (p.head_dim * 1024 + p.v_head_dim) {
             FDK_MFMA_CASE(192v128, 192 * 1024 + 128)

@@ -1,0 +1,483 @@
+// Split-KV paged decode for LARGE q-head groups on one kv head, matrix-core path, gfx950: the shape of latent
+// attention, where 128 q heads share one kv head whose rows hold 576 (K) and 512 (V) values.
+//
+// The kernels of fdk_splitkv_mfma.h give a wavefront one kv head and 16 q heads (the reference's BLOCK_H,
+// python/triton_dist/kernels/nvidia/flash_decode.py:103-109,170-176): with G q heads per kv head the K / V rows are
+// read G / 16 times, and every tile of 16 tokens is copied to LDS once per 16 q heads.  That is the right shape while
+// the memory system is the limit (G <= 16: every row is read once).  At G = 128 it is not: the rows cross the L2 eight
+// times and the matrix cores idle.  Here the wavefronts of a workgroup take DIFFERENT q-head tiles of the SAME kv head
+// and the same tokens: a tile of K / V rows is loaded once by the workgroup (each wavefront loads a quarter of its
+// rows), staged once in LDS, and every wavefront multiplies it with its own 16 q heads.  Two staged tiles alternate,
+// so one barrier per tile is enough: a wavefront writes tile t + 1 only after the barrier of tile t, which every
+// wavefront reaches after it has finished reading tile t - 1 from the same buffer.
+//
+// A workgroup covers kSharedTileHeads = 64 q heads (four wavefronts, each alone on its SIMD with the whole register
+// file: 128 registers of output tile and 72 of Q^T per lane at 576 / 512); a group of 128 is two such workgroups,
+// which the launch places on one XCD (tiles_on_one_xcd).  Same arithmetic per (q head, token) as the other kernels
+// (fdk_splitkv_mfma_body.h): S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with 16x16x16 MFMA
+// and P rounded to the cache dtype; the QK product runs as six interleaved accumulation chains (18 dependent MFMA
+// would wait for each other), and the running maximum of the softmax is a reference that moves rarely, so that the
+// tile loop holds no rescale of the output tile (see move_reference).  16-bit caches; page numbers per tile or per row (PM_TILE, PM_ROW).  How pieces are
+// handed out is shared with the other kernels (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
+#pragma once
+
+#include "fdk_splitkv_mfma.h"
+
+namespace fdk {
+
+namespace {
+
+constexpr int kSharedWaves = 4;                        // wavefronts per workgroup = 16-head tiles per workgroup
+constexpr int kSharedTileHeads = 16 * kSharedWaves;    // q heads of one kv head that a workgroup covers
+
+// REUSE: another workgroup reads the same K / V rows (a group of more than 64 q heads): plain loads, so that the rows
+// stay in the XCD's L2 for it; otherwise the rows are read once and come with the non-temporal hint.
+template <int QDT, int PM, int DK, int DV, int MODE, bool REUSE>
+__global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(const SplitParams p) {
+    using M = Mma<QDT>;
+    using P2 = Pack2<QDT>;
+    using RK = Rows<false, DK>;
+    using RV = Rows<false, DV>;
+    static_assert(PM == PM_TILE || PM == PM_ROW, "page numbers per tile or per row");
+    static_assert(DK % 64 == 0 && DV % 64 == 0, "the LDS swizzle acts on groups of eight 16-byte chunks");
+    constexpr bool kOneSegment = false;        // (fdk_splitkv_mfma_work.h: several head tiles of a kv head go to one XCD)
+    constexpr int kTileHeads = kSharedTileHeads;
+    constexpr int NW = kSharedWaves;
+    constexpr int ES = 2;
+    constexpr int RBK = 2 * DK, RBV = 2 * DV;  // bytes of a staged row
+    constexpr int KS = DK / 32;                // k-steps of the QK product
+    constexpr int DB = DV / 16;                // 16-column blocks of the output
+    constexpr int kTileBytes = kTile * (RBK + RBV);
+    // load instructions of a tile that one wavefront issues, per segment of the rows (Rows<>)
+    constexpr int KS0 = (RK::NJ0 + NW - 1) / NW, KS1 = (RK::NJ1 + NW - 1) / NW;
+    constexpr int VS0 = (RV::NJ0 + NW - 1) / NW, VS1 = (RV::NJ1 + NW - 1) / NW;
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];      // two staged tiles, then the next work item
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int a = lane >> 4;                   // lane group: MFMA k-group / token group
+    const int c = lane & 15;                   // MFMA row/column index
+    const int nh = 1, hl = 0, tix = 0;         // one kv head per workgroup; every wavefront sees every tile
+    int* const s_next = reinterpret_cast<int*>(lds + 2 * kTileBytes);
+
+    auto write_empty_rows = [&](const int b, const int head0, const int heads_here) {
+        for (int idx = lane; idx < heads_here * DV; idx += 64) {
+            const int g = idx / DV, d = idx % DV;
+            const int64_t ob = (int64_t)b * p.out_sb + (int64_t)(head0 + g) * p.out_sh;
+            store_out(p.out, ob + d, 0.f, p.out_dtype);
+            if (d == 0) {
+                if (p.lse) p.lse[(int64_t)b * p.lse_sb + head0 + g] = -INFINITY;
+                if (p.pack_lse) store_out(p.out, ob + DV, -INFINITY, p.out_dtype);
+            }
+        }
+    };
+
+    // One piece: tokens [c_start, min(c_limit, kv_len)) of sequence b for kv head hgb and the q heads
+    // [ht * 64, ht * 64 + 64) of its group; this wavefront's are the 16 from ht * 64 + 16 * wave on.  The partial
+    // results of head g of the 64 go to row prow0 + g * prow_step of the workspace.  (mr: the single-launch form is not
+    // built for this kernel.)
+    auto run_piece = [&](const int b, const int hgb, const int ht, const int c_start, const int c_limit,
+                         const int64_t prow0, const int prow_step, MergeRows /*mr*/) {
+        const int kvh = hgb;
+        const int head_w = ht * kTileHeads + 16 * wave;             // this wavefront's first q head within the group
+        const int heads_here = min(16, p.group - head_w);           // <= 0: the wavefront only helps to load
+        const bool active = heads_here > 0;
+        const int head0 = kvh * p.group + head_w;
+
+        // Q^T, the B operand of S^T = K Q^T: lane (h = c, a) supplies q[h][32 ks + 8 a .. + 7] in k-step ks; 72 registers per
+        // lane at 576 values, kept for the whole piece (read from LDS per tile instead, they doubled the LDS traffic of
+        // the QK product, which is what bounds it).  Columns past the group repeat its last head; their results are
+        // never stored.
+        uint4 qreg[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qreg[ks] = make_uint4(0, 0, 0, 0);
+        if (active) {
+            const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
+                                 (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+        }
+        const ConstI32 tbl = as_const(p.block_table + (int64_t)b * p.tbl_sb);
+        const int pmask = p.page_size - 1;
+        const int kv_len = min(as_const(p.kv_lens)[b], p.max_tokens);
+        if (c_start >= kv_len) {                                    // (the same for every wavefront of the workgroup)
+            if (p.direct && active) write_empty_rows(b, head0, heads_here);
+            return;
+        }
+        const int c_end = min(c_limit, kv_len);
+        const int n_tiles = (c_end - c_start + kTile - 1) / kTile;
+        // the page number of tile t (PM_TILE), or of its row c in every lane (c, any a) (PM_ROW); any t may be asked for
+        auto page_id = [&](int t) {
+            const int tok0 = c_start + t * kTile;
+            if (PM == PM_TILE) return tbl[min(tok0, c_end - 1) >> p.page_shift];
+            const int n = min(tok0 + c, c_end - 1);
+            return tbl[p.page_shift < 0 ? n / p.page_size : n >> p.page_shift];
+        };
+
+        const bool softcap = p.soft_cap > 0.f;
+        const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
+        const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;
+        const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
+        const uint32_t ksp_bytes = (uint32_t)(p.k_sp * ES), vsp_bytes = (uint32_t)(p.v_sp * ES);
+        const uint32_t kst_bytes = (uint32_t)(p.k_st * ES), vst_bytes = (uint32_t)(p.v_st * ES);
+        // rows that the other workgroups of the group read as well stay in the XCD's L2 (plain loads); rows that are
+        // read once come with the non-temporal hint
+        auto load16 = [&](const char* ptr) { return REUSE ? *reinterpret_cast<const uint4*>(ptr) : load_stream16(ptr); };
+
+        struct Tile {                                               // this wavefront's share of a tile, as loaded
+            uint32_t k[KS0 + KS1][4];
+            uint32_t v[VS0 + VS1][4];
+        };
+        // Load instruction j of a segment covers rows j * RPL .. + RPL - 1 (a lane: row j * RPL + lane / LPR, 16 bytes
+        // from byte seg + (lane % LPR) * 16 of the cache row); wavefront w issues the instructions j = w, w + 4, ...
+        // This lane's place within the rows of a load instruction, as a byte offset from the first row (one value per
+        // segment and tensor; everything else about an address of a full tile is wave-uniform or a few lane operations).
+        const uint32_t k_lane0 = (uint32_t)(lane / RK::LPR0) * kst_bytes + (uint32_t)(lane % RK::LPR0) * 16;
+        const uint32_t k_lane1 = (uint32_t)(lane / RK::LPR1) * kst_bytes + (uint32_t)(RK::D0 * ES + (lane % RK::LPR1) * 16);
+        const uint32_t v_lane0 = (uint32_t)(lane / RV::LPR0) * vst_bytes + (uint32_t)(lane % RV::LPR0) * 16;
+        const uint32_t v_lane1 = (uint32_t)(lane / RV::LPR1) * vst_bytes + (uint32_t)(RV::D0 * ES + (lane % RV::LPR1) * 16);
+        // One load: rows first_row .. of the tile at token tok0, this lane's 16 bytes.  CLAMP (the partial last tile of
+        // a piece): rows past the end repeat the last one, which is masked later.
+        // The load instruction of a segment (it has n of them per tile) that this wavefront issues in its slot s.  Where
+        // the wavefronts outnumber the instructions left for the last slot, the surplus wavefronts repeat instructions
+        // of the others (same rows, same place in LDS): every wavefront then runs the same straight-line sequence of
+        // loads and stores, and the waits the compiler puts in front of the stores can count the loads they follow
+        // instead of waiting for all of them.
+        auto slot_instr = [&](int s, int n) {
+            const int j = NW * s + wave;
+            return j < n ? j : j % n;
+        };
+        auto load_rows = [&](auto clamp_tag, int tok0, int32_t pg_id, int first_row, int lane_row, uint32_t lane_off,
+                             uint32_t lane_byte, const char* plane, uint32_t sp_bytes, uint32_t st_bytes) {
+            constexpr bool CLAMP = decltype(clamp_tag)::value;
+            if (PM == PM_TILE && !CLAMP) {
+                // the tile lies in one page: a wave-uniform base plus the lane's offset
+                const int n0 = tok0 + first_row;
+                return load16(plane + ((uint64_t)(uint32_t)pg_id * sp_bytes + (uint64_t)((uint32_t)(n0 & pmask) * st_bytes)) + lane_off);
+            }
+            int n = tok0 + first_row + lane_row;
+            if (CLAMP) n = min(n, c_end - 1);
+            const uint32_t slot = PM == PM_TILE ? (uint32_t)(n & pmask) : (uint32_t)(p.page_shift < 0 ? n % p.page_size : (n & pmask));
+            const uint32_t pg = (uint32_t)(PM == PM_TILE ? pg_id : __shfl(pg_id, n - tok0, 64));
+            return load16(plane + ((uint64_t)pg * sp_bytes + (uint64_t)(slot * st_bytes)) + lane_byte);
+        };
+        auto issue = [&](auto clamp_tag, int t, int32_t pg_id, Tile& rg) {
+            const int tok0 = c_start + t * kTile;
+            int ln = lane;                                  // (as in stage below)
+            asm volatile("" : "+v"(ln));
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                    put(rg.k[s], load_rows(clamp_tag, tok0, pg_id, j * RK::RPL0, ln / RK::LPR0, k_lane0, (ln % RK::LPR0) * 16,
+                                           kplane, ksp_bytes, kst_bytes));
+            }
+#pragma unroll
+            for (int s = 0; s < KS1; ++s) {
+                const int j = slot_instr(s, RK::NJ1);
+                    put(rg.k[KS0 + s], load_rows(clamp_tag, tok0, pg_id, j * RK::RPL1, ln / RK::LPR1, k_lane1,
+                                                 RK::D0 * ES + (ln % RK::LPR1) * 16, kplane, ksp_bytes, kst_bytes));
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                    put(rg.v[s], load_rows(clamp_tag, tok0, pg_id, j * RV::RPL0, ln / RV::LPR0, v_lane0, (ln % RV::LPR0) * 16,
+                                           vplane, vsp_bytes, vst_bytes));
+            }
+#pragma unroll
+            for (int s = 0; s < VS1; ++s) {
+                const int j = slot_instr(s, RV::NJ1);
+                    put(rg.v[VS0 + s], load_rows(clamp_tag, tok0, pg_id, j * RV::RPL1, ln / RV::LPR1, v_lane1,
+                                                 RV::D0 * ES + (ln % RV::LPR1) * 16, vplane, vsp_bytes, vst_bytes));
+            }
+        };
+        // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
+        auto stage = [&](const Tile& rg, char* buf) {
+            char* lk = buf;
+            char* lv = buf + kTile * RBK;
+            // (the lane number through an empty asm: the per-lane parts of the nine store addresses are then computed
+            // here, a few operations each, instead of being kept in registers - or spilled - across the tile loop)
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0)) = get(rg.k[s]);
+            }
+#pragma unroll
+            for (int s = 0; s < KS1; ++s) {
+                const int j = slot_instr(s, RK::NJ1);
+                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1)) =
+                        get(rg.k[KS0 + s]);
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0)) = get(rg.v[s]);
+            }
+#pragma unroll
+            for (int s = 0; s < VS1; ++s) {
+                const int j = slot_instr(s, RV::NJ1);
+                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1)) =
+                        get(rg.v[VS0 + s]);
+            }
+        };
+
+        // Online softmax against a REFERENCE maximum that moves rarely.  The output tile lives in the accumulation
+        // registers, which only the matrix cores reach directly; a rescale by exp2(old max - new max) goes through the
+        // vector ALU, i.e. through copies of all 128 registers, and with the rescale inside the tile loop the compiler
+        // keeps the tile in vector registers for part of every iteration (256 copies per tile, and everything else
+        // spilled).  So the loop over the tiles holds no rescale: probabilities are exp2(logit - m_ref) with a reference
+        // m_ref that may lie up to kSlack below the true running maximum (p <= 2^8, no problem for fp32 sums nor for P
+        // rounded to 16 bits), and a tile whose logits exceed m_ref + kSlack leaves the loop, moves the reference
+        // (move_reference, the rare path) and is done again.  l, the output and the lse are exact whatever the reference
+        // is: lse = m_ref + log2(sum of exp2(logit - m_ref)).
+        constexpr float kSlack = 8.f;
+        float m_ref = -INFINITY, l_run = 0.f;        // for head c; l_run is this lane group's share of the sum
+        float mx_seen = 0.f;                          // the tile maximum that made try_compute give up
+        f32x4_t acc[DB];                              // acc[db][i] = O[h = c][16 db + 4 a + i]
+#pragma unroll
+        for (int db = 0; db < DB; ++db) acc[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        auto move_reference = [&]() {
+            const float m_new = fmaxf(m_ref, mx_seen);               // finite: a tile holds a valid token
+            const float alpha = fast_exp2(m_ref - m_new);            // 0 the first time (m_ref = -inf)
+            l_run *= alpha;
+            // (eight blocks at a time: all 128 registers at once would push everything else out of the vector registers)
+#pragma unroll
+            for (int g = 0; g < DB / 8; ++g) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[8 * g + i] *= alpha;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            m_ref = m_new;
+        };
+
+        // One tile.  False: a logit of the tile exceeds the reference by more than the slack; nothing has been changed.
+        auto try_compute = [&](int t, const char* buf, auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            const int tok0 = c_start + t * kTile;
+            // Where this lane reads its MFMA operands in the staged tile.  The swizzle XORs the low bits of the
+            // 16-byte chunk index with the low bits of the row, so the chunks of one lane are 128 bytes apart within
+            // each class of the low bits: two base addresses for K (k-steps of either parity), four for V (output blocks
+            // modulo four), and constant steps - not one address per operand, which at 18 k-steps and 32 output blocks
+            // would be fifty registers held across the tile loop.
+            //   K operand of k-step ks: row c, chunk 4 ks + a  ->  chunk ^ (c & 7) = 8 (ks >> 1) + ((4 (ks & 1) + a) ^ (c & 7))
+            //   V operand of block db (transposed read): row 4 a + (c >> 2), chunk 2 db + ((c & 3) >> 1)
+            //                                            ->  2 (4 (db >> 2) + ((db & 3) ^ (row & 3))) + ((c & 3) >> 1)
+            const char* lk = buf + c * RBK;
+            const char* k_at[2] = {lk + (((0 + a) ^ (c & 7)) << 4), lk + (((4 + a) ^ (c & 7)) << 4)};
+            const int k4 = c >> 2, cc = c & 3;
+            const int vrow = 4 * a + k4;
+            const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8;
+            const char* v_at[4] = {lv + ((0 ^ (vrow & 3)) << 5), lv + ((1 ^ (vrow & 3)) << 5), lv + ((2 ^ (vrow & 3)) << 5),
+                                   lv + ((3 ^ (vrow & 3)) << 5)};
+            // ---- S^T[token][head] = K Q^T: QG accumulation chains; the K operands of the next QG k-steps are requested
+            // from LDS before the MFMA of the current ones (and no further ahead: every operand held in registers is
+            // one the output tile and the loads under way cannot have) ----
+            constexpr int QG = 6, NQG = KS / QG;
+            static_assert(KS % QG == 0, "k-steps in whole groups");
+            f32x4_t s3[QG];
+#pragma unroll
+            for (int i = 0; i < QG; ++i) s3[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            uint4 ka[2][QG];
+            auto read_qk = [&](int g, int to) {
+#pragma unroll
+                for (int i = 0; i < QG; ++i) {
+                    const int ks = g * QG + i;
+                    ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + (ks >> 1) * 128);
+                }
+            };
+            read_qk(0, 0);
+#pragma unroll
+            for (int g = 0; g < NQG; ++g) {
+                if (g + 1 < NQG) read_qk(g + 1, (g + 1) & 1);
+#pragma unroll
+                for (int i = 0; i < QG; ++i) s3[i] = M::qk(ka[g & 1][i], qreg[g * QG + i], s3[i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            f32x4_t s = s3[0];
+#pragma unroll
+            for (int i = 1; i < QG; ++i) s += s3[i];
+            float sv[4] = {s.x, s.y, s.z, s.w};
+            if (softcap) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * p.sm_scale, p.soft_cap, inv_cap) * kLog2e;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sv[i] *= p.scale_log2;
+            }
+            if (MASKED) {                         // the last tile of the piece may be partial
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (tok0 + 4 * a + i >= c_end) sv[i] = -INFINITY;
+            }
+            float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));          // finite: token tok0 is valid
+            if (__builtin_amdgcn_ballot_w64(mx > m_ref + kSlack) != 0) {
+                mx_seen = mx;
+                return false;
+            }
+            float pr[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pr[i] = fast_exp2(sv[i] - m_ref);
+            l_run += (pr[0] + pr[1]) + (pr[2] + pr[3]);
+            // P^T as B operand, rounded to the cache dtype as the reference does before its second dot (flash_decode.py:230)
+            const uint2 pb = make_uint2(P2::pack(pr[0], pr[1]), P2::pack(pr[2], pr[3]));
+            // ---- O^T[d][head] += V^T P^T ----
+            constexpr int VG = 16, NVG = DB / VG;
+            static_assert(DB % VG == 0, "output blocks in whole groups");
+            uint2 va[2][VG];
+            auto read_v = [&](int g, int to) {
+#pragma unroll
+                for (int i = 0; i < VG; ++i)
+                    va[to][i] = M::read_tr(v_at[(g * VG + i) & 3] + ((g * VG + i) >> 2) * 128);
+            };
+            read_v(0, 0);
+#pragma unroll
+            for (int g = 0; g < NVG; ++g) {
+                if (g + 1 < NVG) read_v(g + 1, (g + 1) & 1);
+#pragma unroll
+                for (int i = 0; i < VG; ++i) acc[g * VG + i] = M::pv(va[g & 1][i], pb, acc[g * VG + i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            return true;
+        };
+
+        // ---- the tiles of the piece: the loads of tiles t + 1 and t + 2 are under way while all wavefronts work on tile t
+        // (two register tiles by the parity of t; the memory system's latency is longer than the arithmetic of one tile).
+        // Page numbers are requested two tiles further ahead, BEFORE the rows of the tile in between: vector loads return
+        // in order, so waiting for a number then never waits for rows requested after it.
+        // (A wavefront that leaves the inner loop to move its reference does so after the tile's barrier and comes back for
+        // the next tile: every wavefront passes exactly one barrier per tile.) ----
+        {
+            Tile rg_even, rg_odd;
+            const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
+            auto issue_tile = [&](int t, int32_t pg_id, Tile& rg) {
+                if (t < n_full) issue(BoolTag<false>(), t, pg_id, rg);
+                else if (t < n_tiles) issue(BoolTag<true>(), t, pg_id, rg);
+            };
+            int32_t pg_even = page_id(0), pg_odd = page_id(1);
+            issue_tile(0, pg_even, rg_even);
+            pg_even = page_id(2);
+            issue_tile(1, pg_odd, rg_odd);
+            pg_odd = page_id(3);
+            // tile t up to its barrier: stage it, request the rows of tile t + 2 into the registers it came from
+            auto stage_and_issue = [&](int t, Tile& rg, int32_t& pg) {
+                stage(rg, lds + (t & 1) * kTileBytes);              // waits for this wavefront's loads of tile t
+                issue_tile(t + 2, pg, rg);
+                pg = page_id(t + 4);
+                // tile t is staged; tile t - 1 has been read by everyone.  (The barrier waits for this wavefront's LDS
+                // operations only: __syncthreads() would also wait for the rows just requested from memory, i.e. for the
+                // very loads that are meant to be under way during the arithmetic.)
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            };
+            int t = 0;
+            for (;;) {
+                bool gave_up = false;
+                for (; t < n_full; ++t) {
+                    if (t & 1) stage_and_issue(t, rg_odd, pg_odd);
+                    else stage_and_issue(t, rg_even, pg_even);
+                    if (active && !try_compute(t, lds + (t & 1) * kTileBytes, BoolTag<false>())) {
+                        gave_up = true;
+                        break;
+                    }
+                }
+                if (!gave_up) break;
+                do move_reference(); while (!try_compute(t, lds + (t & 1) * kTileBytes, BoolTag<false>()));
+                ++t;
+            }
+            if (n_full < n_tiles) {                                 // the partial last tile
+                if (n_full & 1) stage_and_issue(n_full, rg_odd, pg_odd);
+                else stage_and_issue(n_full, rg_even, pg_even);
+                if (active) {
+                    while (!try_compute(n_full, lds + (n_full & 1) * kTileBytes, BoolTag<true>())) move_reference();
+                }
+            }
+        }
+        if (!active) return;
+
+        // ---- this wavefront's 16 heads are its own: no merge across wavefronts, results go out from the registers ----
+        l_run += __shfl_xor(l_run, 16, 64);
+        l_run += __shfl_xor(l_run, 32, 64);
+        if (c < heads_here) {
+            const int hq = head0 + c;
+            const float norm = fast_rcp(l_run);                     // > 0: the piece holds a token
+            const float lse_nat = (m_ref + fast_log2(l_run)) * kLn2;
+            const int64_t prow = prow0 + (int64_t)(16 * wave + c) * prow_step;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const float4 o = make_float4(acc[db].x * norm, acc[db].y * norm, acc[db].z * norm, acc[db].w * norm);
+                const int d0 = 16 * db + 4 * a;
+                if (p.direct) store_out4(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0, o, p.out_dtype);
+                else *reinterpret_cast<float4*>(p.part_o + prow * DV + d0) = o;
+            }
+            if (a == 0) {
+                if (p.direct) {
+                    if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
+                    if (p.pack_lse) store_out(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + DV, lse_nat, p.out_dtype);
+                } else {
+                    p.part_lse[prow] = lse_nat;
+                }
+            }
+        }
+    };   // run_piece
+
+#include "fdk_splitkv_mfma_work.h"
+}
+
+// Launch of the shared-tile kernels.  The plan counts head tiles of kSharedTileHeads q heads and one kv head per
+// workgroup for them (mfma_tile_heads, mfma_kv_heads_per_wg).
+template <int QDT, int DK, int DV, int MODE>
+int launch_shared(const SplitParams& p_in, hipStream_t stream) {
+    if (mfma_work_mode(p_in) != MODE || p_in.fused || p_in.probe || p_in.hg_per_wg != 1 || p_in.tile_heads != kSharedTileHeads)
+        return (int)hipErrorInvalidValue;
+    constexpr int kTileBytes = 2 * kTile * (DK + DV);
+    SplitParams p = p_in;
+    p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
+    p.hg_blocks = p.hkv;
+    const size_t lds_bytes = 2 * (size_t)kTileBytes + 16;
+    const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
+    p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
+    // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
+    // than there are pieces: every workgroup of the queue has to take one, or it would not be counted among the
+    // finished ones and the queue's counters would not be put back to zero)
+    const int resident = min(p.num_cus > 0 ? p.num_cus : 256, p.total_items);
+    p.persistent = MODE == WM_QUEUE ? 1 : 0;
+    const unsigned units = (unsigned)(p.hg_blocks * p.head_tiles);
+    const dim3 grid = p.balanced ? dim3(units, (unsigned)p.workgroups / units)
+                    : p.persistent ? dim3((unsigned)resident)
+                                   : dim3(units, (unsigned)p.num_splits, (unsigned)p.batch);
+    const dim3 block(64 * kSharedWaves);
+    p.shares = (int32_t)grid.y;
+    p.grid_x = (int32_t)grid.x;
+    p.wavefronts = kSharedWaves;
+    const bool reuse = p.head_tiles > 1;
+#define FDK_SHARED_LAUNCH(PMV, RU)                                                                                        \
+    do {                                                                                                                  \
+        const hipError_t e = hipFuncSetAttribute(                                                                         \
+            reinterpret_cast<const void*>(&splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU>),                       \
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);                                                  \
+        if (e != hipSuccess) return (int)e;                                                                               \
+        hipLaunchKernelGGL((splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU>), grid, block, lds_bytes, stream, p);  \
+    } while (0)
+    if (pm == PM_TILE) {
+        if (reuse) FDK_SHARED_LAUNCH(PM_TILE, true);
+        else FDK_SHARED_LAUNCH(PM_TILE, false);
+    } else {
+        if (reuse) FDK_SHARED_LAUNCH(PM_ROW, true);
+        else FDK_SHARED_LAUNCH(PM_ROW, false);
+    }
+#undef FDK_SHARED_LAUNCH
+    return (int)hipGetLastError();
+}
+
+template <int DK, int DV, int MODE>
+int launch_mfma_shared(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    if (kv_dtype != q_dtype) return (int)hipErrorInvalidValue;
+    return q_dtype == FDK_BF16 ? launch_shared<FDK_BF16, DK, DV, MODE>(p, stream) : launch_shared<FDK_FP16, DK, DV, MODE>(p, stream);
+}
+
+}  // namespace
+
+}  // namespace fdk
