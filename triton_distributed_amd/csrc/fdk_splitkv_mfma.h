@@ -303,8 +303,10 @@ __global__ __launch_bounds__(rows2_max_threads(DK, DV)) void splitkv_mfma_rows2_
 // queue keeps every compute unit busy until the end.
 inline bool mfma_runs_as_queue(const SplitParams& p) {
     const int hg_per_wg = (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) ? 1 : p.hg_per_wg;
-    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + 15) / 16);
-    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);     // two 4-wave workgroups fit a compute unit
+    const int tile_heads = p.tile_heads > 16 ? p.tile_heads : 16;       // q heads of a kv head per workgroup
+    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + tile_heads - 1) / tile_heads);
+    // two 4-wave workgroups fit a compute unit; of the kernels that cover 64 q heads per workgroup, one
+    const int resident = (tile_heads > 16 ? 1 : 2) * (p.num_cus > 0 ? p.num_cus : 256);
     return p.counters != nullptr && !p.direct && !p.balanced && items > resident;
 }
 inline int mfma_work_mode(const SplitParams& p) { return p.balanced ? WM_SHARES : mfma_runs_as_queue(p) ? WM_QUEUE : WM_ONE; }

@@ -19,8 +19,10 @@ FDK_DECLARE_MFMA(576v512_shared) // ... large q-head groups: wavefronts share th
 // (the same rule as mfma_work_mode in the kernel header, which this file does not include)
 static int work_mode_of(const SplitParams& p) {
     const int hg_per_wg = (p.hg_per_wg < 1 || p.hkv % p.hg_per_wg) ? 1 : p.hg_per_wg;
-    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + 15) / 16);
-    const int resident = 2 * (p.num_cus > 0 ? p.num_cus : 256);
+    const int tile_heads = p.tile_heads > 16 ? p.tile_heads : 16;       // q heads of a kv head per workgroup
+    const int64_t items = (int64_t)p.batch * p.num_splits * (p.hkv / hg_per_wg) * ((p.group + tile_heads - 1) / tile_heads);
+    // two 4-wave workgroups fit a compute unit; of the kernels that cover 64 q heads per workgroup, one
+    const int resident = (tile_heads > 16 ? 1 : 2) * (p.num_cus > 0 ? p.num_cus : 256);
     return p.balanced ? 2 : (p.counters != nullptr && !p.direct && items > resident) ? 1 : 0;
 }
 
