@@ -6,19 +6,21 @@
 // read G / 16 times, and every tile of 16 tokens is copied to LDS once per 16 q heads.  That is the right shape while
 // the memory system is the limit (G <= 16: every row is read once).  At G = 128 it is not: the rows cross the L2 eight
 // times and the matrix cores idle.  Here the wavefronts of a workgroup take DIFFERENT q-head tiles of the SAME kv head
-// and the same tokens: a tile of K / V rows is loaded once by the workgroup (each wavefront loads a quarter of its
+// and the same tokens: a tile of K / V rows is loaded once by the workgroup (each wavefront loads its share of the
 // rows), staged once in LDS, and every wavefront multiplies it with its own 16 q heads.  Two staged tiles alternate,
 // so one barrier per tile is enough: a wavefront writes tile t + 1 only after the barrier of tile t, which every
 // wavefront reaches after it has finished reading tile t - 1 from the same buffer.
 //
-// A workgroup covers kSharedTileHeads = 64 q heads (four wavefronts, each alone on its SIMD with the whole register
-// file: 128 registers of output tile and 72 of Q^T per lane at 576 / 512); a group of 128 is two such workgroups,
-// which the launch places on one XCD (tiles_on_one_xcd).  Same arithmetic per (q head, token) as the other kernels
-// (fdk_splitkv_mfma_body.h): S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with 16x16x16 MFMA
-// and P rounded to the cache dtype; the QK product runs as six interleaved accumulation chains (18 dependent MFMA
-// would wait for each other), and the running maximum of the softmax is a reference that moves rarely, so that the
-// tile loop holds no rescale of the output tile (see move_reference).  16-bit caches; page numbers per tile or per row (PM_TILE, PM_ROW).  How pieces are
-// handed out is shared with the other kernels (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
+// A workgroup covers kSharedTileHeads = 64 q heads with eight wavefronts: two per tile of 16 q heads, each of which
+// forms the tile's logits and softmax for itself and accumulates one half of the output columns (64 accumulation
+// registers per lane at 512 values; Q^T takes 72 more), two wavefronts per SIMD.  A group of 128 q heads is two such
+// workgroups, which the launch places on one XCD (tiles_on_one_xcd).  Same arithmetic per (q head, token) as the other
+// kernels (fdk_splitkv_mfma_body.h): S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with
+// 16x16x16 MFMA and P rounded to the cache dtype; the QK product runs as six interleaved accumulation chains (18
+// dependent MFMA would wait for each other), and the running maximum of the softmax is a reference that moves rarely,
+// so that the tile loop holds no rescale of the output tile (see move_reference).  16-bit caches; page numbers per tile
+// or per row (PM_TILE, PM_ROW).  How pieces are handed out is shared with the other kernels
+// (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
 #pragma once
 
 #include "fdk_splitkv_mfma.h"
@@ -27,8 +29,10 @@ namespace fdk {
 
 namespace {
 
-constexpr int kSharedWaves = 4;                        // wavefronts per workgroup = 16-head tiles per workgroup
-constexpr int kSharedTileHeads = 16 * kSharedWaves;    // q heads of one kv head that a workgroup covers
+constexpr int kSharedWaves = 8;                        // wavefronts per workgroup
+constexpr int kSharedColSplit = 2;                     // wavefronts that share a tile of 16 q heads, each with 1 / kSharedColSplit
+                                                       // of the output columns (both form the tile's logits and softmax)
+constexpr int kSharedTileHeads = 16 * kSharedWaves / kSharedColSplit;    // q heads of one kv head that a workgroup covers
 
 // REUSE: another workgroup reads the same K / V rows (a group of more than 64 q heads): plain loads, so that the rows
 // stay in the XCD's L2 for it; otherwise the rows are read once and come with the non-temporal hint.
@@ -46,7 +50,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr int ES = 2;
     constexpr int RBK = 2 * DK, RBV = 2 * DV;  // bytes of a staged row
     constexpr int KS = DK / 32;                // k-steps of the QK product
-    constexpr int DB = DV / 16;                // 16-column blocks of the output
+    constexpr int CS = kSharedColSplit;
+    constexpr int DB = DV / 16 / CS;           // 16-column blocks of the output that this wavefront holds
     constexpr int kTileBytes = kTile * (RBK + RBV);
     // load instructions of a tile that one wavefront issues, per segment of the rows (Rows<>)
     constexpr int KS0 = (RK::NJ0 + NW - 1) / NW, KS1 = (RK::NJ1 + NW - 1) / NW;
@@ -59,6 +64,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     const int a = lane >> 4;                   // lane group: MFMA k-group / token group
     const int c = lane & 15;                   // MFMA row/column index
     const int nh = 1, hl = 0, tix = 0;         // one kv head per workgroup; every wavefront sees every tile
+    const int wtile = wave / CS;               // this wavefront's tile of 16 q heads within the workgroup's
+    const int whalf = wave % CS;               // ... and its part of the output columns
     int* const s_next = reinterpret_cast<int*>(lds + 2 * kTileBytes);
 
     auto write_empty_rows = [&](const int b, const int head0, const int heads_here) {
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     auto run_piece = [&](const int b, const int hgb, const int ht, const int c_start, const int c_limit,
                          const int64_t prow0, const int prow_step, MergeRows /*mr*/) {
         const int kvh = hgb;
-        const int head_w = ht * kTileHeads + 16 * wave;             // this wavefront's first q head within the group
+        const int head_w = ht * kTileHeads + 16 * wtile;            // this wavefront's first q head within the group
         const int heads_here = min(16, p.group - head_w);           // <= 0: the wavefront only helps to load
         const bool active = heads_here > 0;
         const int head0 = kvh * p.group + head_w;
@@ -102,7 +109,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         const int pmask = p.page_size - 1;
         const int kv_len = min(as_const(p.kv_lens)[b], p.max_tokens);
         if (c_start >= kv_len) {                                    // (the same for every wavefront of the workgroup)
-            if (p.direct && active) write_empty_rows(b, head0, heads_here);
+            if (p.direct && active && whalf == 0) write_empty_rows(b, head0, heads_here);
             return;
         }
         const int c_end = min(c_limit, kv_len);
@@ -192,34 +199,36 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             }
         };
         // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
+        // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
         auto stage = [&](const Tile& rg, char* buf) {
             char* lk = buf;
             char* lv = buf + kTile * RBK;
-            // (the lane number through an empty asm: the per-lane parts of the nine store addresses are then computed
-            // here, a few operations each, instead of being kept in registers - or spilled - across the tile loop)
+            // (the lane number through an empty asm: the per-lane parts of the store addresses are then computed here, a
+            // few operations each, instead of being kept in registers - or spilled, and a spill reload waits for every
+            // load under way - across the tile loop)
             int ln = lane;
             asm volatile("" : "+v"(ln));
 #pragma unroll
             for (int s = 0; s < KS0; ++s) {
                 const int j = slot_instr(s, RK::NJ0);
-                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0)) = get(rg.k[s]);
+                *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0)) = get(rg.k[s]);
             }
 #pragma unroll
             for (int s = 0; s < KS1; ++s) {
                 const int j = slot_instr(s, RK::NJ1);
-                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1)) =
-                        get(rg.k[KS0 + s]);
+                *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1)) =
+                    get(rg.k[KS0 + s]);
             }
 #pragma unroll
             for (int s = 0; s < VS0; ++s) {
                 const int j = slot_instr(s, RV::NJ0);
-                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0)) = get(rg.v[s]);
+                *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0)) = get(rg.v[s]);
             }
 #pragma unroll
             for (int s = 0; s < VS1; ++s) {
                 const int j = slot_instr(s, RV::NJ1);
-                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1)) =
-                        get(rg.v[VS0 + s]);
+                *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1)) =
+                    get(rg.v[VS0 + s]);
             }
         };
 
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             const char* k_at[2] = {lk + (((0 + a) ^ (c & 7)) << 4), lk + (((4 + a) ^ (c & 7)) << 4)};
             const int k4 = c >> 2, cc = c & 3;
             const int vrow = 4 * a + k4;
-            const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8;
+            const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8 + whalf * (DB / 4) * 128;   // (+ this wavefront's columns)
             const char* v_at[4] = {lv + ((0 ^ (vrow & 3)) << 5), lv + ((1 ^ (vrow & 3)) << 5), lv + ((2 ^ (vrow & 3)) << 5),
                                    lv + ((3 ^ (vrow & 3)) << 5)};
             // ---- S^T[token][head] = K Q^T: QG accumulation chains; the K operands of the next QG k-steps are requested
@@ -325,7 +334,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // P^T as B operand, rounded to the cache dtype as the reference does before its second dot (flash_decode.py:230)
             const uint2 pb = make_uint2(P2::pack(pr[0], pr[1]), P2::pack(pr[2], pr[3]));
             // ---- O^T[d][head] += V^T P^T ----
-            constexpr int VG = 16, NVG = DB / VG;
+            constexpr int VG = DB < 16 ? DB : 16, NVG = DB / VG;
             static_assert(DB % VG == 0, "output blocks in whole groups");
             uint2 va[2][VG];
             auto read_v = [&](int g, int to) {
@@ -404,15 +413,15 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             const int hq = head0 + c;
             const float norm = fast_rcp(l_run);                     // > 0: the piece holds a token
             const float lse_nat = (m_ref + fast_log2(l_run)) * kLn2;
-            const int64_t prow = prow0 + (int64_t)(16 * wave + c) * prow_step;
+            const int64_t prow = prow0 + (int64_t)(16 * wtile + c) * prow_step;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 const float4 o = make_float4(acc[db].x * norm, acc[db].y * norm, acc[db].z * norm, acc[db].w * norm);
-                const int d0 = 16 * db + 4 * a;
+                const int d0 = 16 * (whalf * DB + db) + 4 * a;
                 if (p.direct) store_out4(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + d0, o, p.out_dtype);
                 else *reinterpret_cast<float4*>(p.part_o + prow * DV + d0) = o;
             }
-            if (a == 0) {
+            if (a == 0 && whalf == 0) {
                 if (p.direct) {
                     if (p.lse) p.lse[(int64_t)b * p.lse_sb + hq] = lse_nat;
                     if (p.pack_lse) store_out(p.out, (int64_t)b * p.out_sb + (int64_t)hq * p.out_sh + DV, lse_nat, p.out_dtype);
