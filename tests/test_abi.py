@@ -650,6 +650,13 @@ def test_plans_of_wide_rows_keep_to_what_a_compute_unit_holds():
     assert _plan(_dims(192, 128, **big)).kv_heads_per_wg == 8
     p = _plan(_dims(576, 512, **big))
     assert p.kv_heads_per_wg == 2 and p.num_splits == 1
+    # large q-head groups on one kv head of 576 + 512 values: one kv head and 64 q heads per workgroup (the kernels whose
+    # wavefronts share the staged tiles), so 32 sequences x 128 q heads are 64 units and split four ways on 256 compute units
+    mla = _dims(576, 512, batch=32, num_q_heads=128, num_kv_heads=1, max_kv_len=4096, min_kv_len=4096, q_stride_b=128 * 576,
+                k_stride_page=16 * 576, k_stride_tok=576, v_stride_page=16 * 512, v_stride_tok=512, out_stride_b=128 * 512,
+                lse_stride_b=128)
+    p = _plan(mla)
+    assert p.kv_heads_per_wg == 1 and p.num_splits == 4 and not p.balanced
     # streaming estimates count the K and the V row: a (192, 128) cache streams 5/6 of what a (192, 192) cache does
     a, b = _plan(_dims(192, 192, batch=8, max_kv_len=4096)), _plan(_dims(192, 128, batch=8, max_kv_len=4096))
     assert a.num_splits >= 1 and b.num_splits >= 1

@@ -56,8 +56,6 @@ struct SplitParams {
     int32_t grid_x;                 // gridDim.x
     int32_t wavefronts;             // blockDim.x / 64
     int32_t rows_per_slot, heads_per_tile;   // balanced mode: partial rows per slot, q heads per tile (<= tile_heads)
-    int32_t tile_heads;             // q heads of a kv head that one workgroup covers: 16 (an MFMA tile), or 64 in the
-                                    // kernels whose wavefronts share the staged tiles (fdk_splitkv_mfma_shared.h)
     int32_t piece_cost;             // balanced mode: granules a sequence counts for on top of its own
     int32_t tune_wavefronts, tune_buffers;   // 0: chosen by the launcher; else the caller's override (measurements)
     int32_t* length_feedback;       // set where this kernel ends the call: {min, max of the clamped kv_lens, epoch, batch} goes here
@@ -73,6 +71,8 @@ struct SplitParams {
     float scale_log2;               // sm_scale * log2(e)
     float soft_cap;                 // > 0: on (applied to natural-unit logits)
     float sm_scale;
+    int32_t tile_heads;             // q heads of a kv head that one workgroup covers: 16 (an MFMA tile), or 64 in the
+                                    // kernels whose wavefronts share the staged tiles (fdk_splitkv_mfma_shared.h)
 };
 
 struct CombineParams {

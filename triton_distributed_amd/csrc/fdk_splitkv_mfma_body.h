@@ -33,6 +33,7 @@
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int kTileHeads = 16;             // q heads per head tile: the 16 columns of an MFMA tile
+    constexpr bool kFirstPieceStraight = true; // (fdk_splitkv_mfma_work.h)
     const int a = lane >> 4;                   // lane group: MFMA k-group / token group
     const int c = lane & 15;                   // MFMA row/column index
     const int lrow = lane / LPR;               // row of this lane within a load

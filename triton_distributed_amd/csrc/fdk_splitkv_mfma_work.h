@@ -1,7 +1,8 @@
 // How the pieces of a call are handed out to the workgroups of the matrix-core split-KV kernels: the second half of
 // each kernel's body (the kernel definitions include this file after they have defined run_piece, write_empty_rows
 // and: p, lane, wave, nh = kv heads per workgroup, hl = this wavefront's kv head within the block, tix = its index among
-// the wavefronts of that head, s_next = an int in LDS, kTileHeads = q heads per head tile, kOneSegment, MODE).
+// the wavefronts of that head, s_next = an int in LDS, kTileHeads = q heads per head tile, kOneSegment, MODE,
+// kFirstPieceStraight = whether a share's first piece gets straight-line code of its own, see below).
     // ---- work distribution --------------------------------------------------------------------------------------
     // Chunk mode: item -> (sequence, split, kv-head block, q-head tile), partial row (b, head, split); one item per
     // workgroup, or (persistent) a fixed set of workgroups that pull items from a queue: counters[0] is its head,
@@ -241,13 +242,23 @@
             run += __builtin_amdgcn_readlane(incl, 63);
         }
         int piece_end = 0;
-        const Piece first = piece_of(piece_end);
-        if (first.c_limit > first.c_start) run_piece(first.pb, first.hgb, first.ht, first.c_start, first.c_limit, first.prow0, 1, first.mr);
-        if (!next_piece(first, piece_end)) return;
-        for (;;) {
-            __syncthreads();                                          // the LDS scratch is reused by the next piece
-            const Piece pp = piece_of(piece_end);
-            if (pp.c_limit > pp.c_start) run_piece(pp.pb, pp.hgb, pp.ht, pp.c_start, pp.c_limit, pp.prow0, 1, pp.mr);
-            if (!next_piece(pp, piece_end)) return;
+        if constexpr (kFirstPieceStraight) {
+            const Piece first = piece_of(piece_end);
+            if (first.c_limit > first.c_start) run_piece(first.pb, first.hgb, first.ht, first.c_start, first.c_limit, first.prow0, 1, first.mr);
+            if (!next_piece(first, piece_end)) return;
+            for (;;) {
+                __syncthreads();                                      // the LDS scratch is reused by the next piece
+                const Piece pp = piece_of(piece_end);
+                if (pp.c_limit > pp.c_start) run_piece(pp.pb, pp.hgb, pp.ht, pp.c_start, pp.c_limit, pp.prow0, 1, pp.mr);
+                if (!next_piece(pp, piece_end)) return;
+            }
+        } else {
+            // (kernels whose piece needs every register: one copy of it, in the loop)
+            for (;;) {
+                const Piece pp = piece_of(piece_end);
+                if (pp.c_limit > pp.c_start) run_piece(pp.pb, pp.hgb, pp.ht, pp.c_start, pp.c_limit, pp.prow0, 1, pp.mr);
+                if (!next_piece(pp, piece_end)) return;
+                __syncthreads();                                      // the LDS scratch is reused by the next piece
+            }
         }
     }
