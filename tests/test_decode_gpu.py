@@ -320,13 +320,13 @@ def test_two_segment_head_dims_in_every_plan(cuda_device, dims, page):
     torch.testing.assert_close(lse_m, l2 + math.log(2.0), atol=1e-4, rtol=0)
 
 
-@pytest.mark.parametrize("seed", list(range(18)))
+@pytest.mark.parametrize("seed", list(range(30)))
 def test_two_segment_head_dims_random_shapes(cuda_device, seed):
     g = torch.Generator().manual_seed(4000 + seed)
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
     dims = TWO_SEGMENT_DIMS[seed % 3]
     hkv = [1, 2, 3, 4, 8][r(0, 4)]
-    group = [1, 2, 4, 7, 8, 16, 20, 40][r(0, 7)]
+    group = [1, 2, 4, 7, 8, 16, 20, 40, 64, 100, 128][r(0, 10)]
     page = [1, 2, 5, 8, 16, 32, 48, 128][r(0, 7)]
     batch = r(1, 20)
     top = [60, 700, 5000][r(0, 2)]
@@ -353,13 +353,14 @@ def test_two_segment_head_dims_random_shapes(cuda_device, seed):
            ref_tol=4e-2 if scale > dims[0] ** -0.5 else None)
 
 
-@pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
-def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(cuda_device, dims):
-    """A captured call (the kernels of the widest rows ask for more LDS than the default limit at launch) replayed on
-    changed q and lengths, and the entry point that allocates nothing, against the eager call."""
+@pytest.mark.parametrize("dims,heads", [(d, (32, 2)) for d in TWO_SEGMENT_DIMS] + [((576, 512), (128, 1))])
+def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(cuda_device, dims, heads):
+    """A captured call (the kernels of the widest rows ask for more LDS than the default limit at launch; 128 q heads on one
+    kv head: the kernels whose wavefronts share the staged tiles) replayed on changed q and lengths, and the entry point
+    that allocates nothing, against the eager call."""
     dk, dv = dims
     g = torch.Generator().manual_seed(dk * 3 + dv)
-    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, [2500] * 4, (32, 2), 16, torch.bfloat16, 31)   # pages for every length below
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, [2500] * 4, heads, 16, torch.bfloat16, 31)   # pages for every length below
     lens_t.copy_(_lens_t([2500, 1, 900, 1800], cuda_device))
     scale = dk ** -0.5
     call = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500)
