@@ -174,6 +174,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             const int tok0 = c_start + t * kTile;
             int ln = lane;                                  // (as in stage below)
             asm volatile("" : "+v"(ln));
+            ln &= 63;                                       // (known to the compiler again: a row of 64 lanes is one row)
 #pragma unroll
             for (int s = 0; s < KS0; ++s) {
                 const int j = slot_instr(s, RK::NJ0);
@@ -209,6 +210,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // load under way - across the tile loop)
             int ln = lane;
             asm volatile("" : "+v"(ln));
+            ln &= 63;                                       // (known to the compiler again: a row of 64 lanes is one row)
 #pragma unroll
             for (int s = 0; s < KS0; ++s) {
                 const int j = slot_instr(s, RK::NJ0);
