@@ -529,11 +529,11 @@ def main():
         # further pools: same pages, different (seeded) contents - the access pattern is identical
         g = torch.Generator(device=dev).manual_seed(inp.cfg.seed + 100 * r)
         if inp.cfg.kv_dtype == "fp8_e4m3":
-            mk = lambda: torch.randint(0, 120, inp.k_cache.shape, generator=g, device=dev, dtype=torch.uint8).view(
-                torch.float8_e4m3fn)
+            mk = lambda like=inp.k_cache: torch.randint(0, 120, like.shape, generator=g, device=dev,
+                                                        dtype=torch.uint8).view(torch.float8_e4m3fn)
         else:
             mk = lambda like=inp.k_cache: torch.randn(like.shape, generator=g, device=dev, dtype=like.dtype)
-        pools.append((mk(), mk(inp.v_cache) if inp.cfg.kv_dtype != "fp8_e4m3" else mk()))
+        pools.append((mk(), mk(inp.v_cache)))
     def prepare_all(pp):
         return [tda.prepare_decode(inp.q, k, v, inp.block_table, inp.kv_lens, inp.sm_scale, k_scale=inp.k_scale,
                                    v_scale=inp.v_scale, kv_split=args.kv_split, algo=args.algo, always_workspace=True,

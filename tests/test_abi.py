@@ -628,8 +628,8 @@ def test_head_dims_of_two_segments_and_v_rows_of_their_own_length():
     assert _decode_rc(a) == 0
     a.workspace_bytes = need - 1
     assert _decode_rc(a) == _lib.FDK_EWORKSPACE
-    # built for 16-bit caches on the matrix-core path, without the single-launch form
-    assert _decode_rc(_dims(192, 192, kv_dtype=_lib.FDK_FP8_E4M3)) == _lib.FDK_EUNSUPPORTED
+    # built on the matrix-core path, without the single-launch form
+    assert _decode_rc(_dims(192, 192, kv_dtype=_lib.FDK_FP8_E4M3, k_stride_page=16 * 8 * 192, v_stride_page=16 * 8 * 192)) == 0   # fp8 caches are built
     assert _decode_rc(_dims(192, 192, algo=_lib.FDK_ALGO_VALU)) == _lib.FDK_EUNSUPPORTED
     assert _decode_rc(_dims(192, 192, flags=_lib.FDK_FLAG_DRY_RUN | _lib.FDK_FLAG_SINGLE_LAUNCH)) == _lib.FDK_EUNSUPPORTED
     assert _plan(_dims(192, 128)).algo == _lib.FDK_ALGO_MFMA

@@ -434,15 +434,57 @@ def test_large_groups_on_one_kv_head_share_the_staged_tiles(cuda_device, heads, 
     torch.testing.assert_close(packed[live][..., 512].float(), lse_a[live], atol=3e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
+@pytest.mark.parametrize("heads,page", [((32, 8), 16), ((16, 2), 4), ((40, 1), 64), ((128, 1), 16)])
+def test_two_segment_head_dims_with_an_fp8_cache(cuda_device, dims, heads, page):
+    """e4m3 caches with per-kv-head scales behind rows of two segments: exact dequantisation (the decode over the
+    dequantised cache) and the K scale folded into the logit scale, through a single pass, chunks and equal shares; large
+    groups run with tiles of 16 q heads here."""
+    dk, dv = dims
+    hq, hkv = heads
+    g = torch.Generator().manual_seed(dk + hq + page)
+    lens = [int(x) for x in torch.randint(1, 1800, (5,), generator=g)]
+    lens[1] = 0
+    q, k16, v16, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, heads, page, torch.bfloat16, 900 + hq + page)
+    k16[-1], v16[-1] = 0, 0                          # (the page of NaN does not quantise)
+    k8, ks = wl.quantize_kv_fp8(k16)
+    v8, vs = wl.quantize_kv_fp8(v16)
+    k8.view(torch.uint8)[-1] = 0x7F                  # unused table columns still point at NaN (0x7F in e4m3)
+    v8.view(torch.uint8)[-1] = 0x7F
+    kd, vd = ofp8.dequant_per_head(k8, ks), ofp8.dequant_per_head(v8, vs)
+    scale = dk ** -0.5
+    live = [i for i, n in enumerate(lens) if n > 0]
+    plan = tda.get_split_kv_plan(q, k8, v8, table, lens_t, scale)
+    assert plan.algo == "mfma"
+    for tag, kw in (("auto", {}), ("single pass", dict(kv_split=1)), ("3 chunks", dict(kv_split=3)), ("equal shares", dict(force_balanced=True)),
+                    ("folded", dict(fp8_fold_k_scale=True))):
+        out, lse = tda.flash_decode(q, k8, v8, table, lens_t, scale, k_scale=ks, v_scale=vs, **kw)
+        torch.cuda.synchronize()
+        assert out.shape == (len(lens), hq, dv)
+        assert float(out[1].abs().max()) == 0 and bool((lse[1] == -math.inf).all()), tag
+        name = f"fp8 dims={dims} heads={heads} P={page} {tag}"
+        ll = [lens[i] for i in live]
+        if tag != "folded":
+            _check(out[live], lse[live], q[live], k8, v8, table[live], ll, scale, ref_kv=(kd, vd), tag=name)
+            continue
+        # the folded form evaluates the cache exactly: the standard bars hold against k8 * k_scale without the 16-bit
+        # rounding of K, and lse is within 5e-3 of the dequantise-then-decode definition (as for one-segment rows)
+        assert torch.isfinite(out.float()).all() and torch.isfinite(lse[live]).all(), name
+        o64, l64 = cf.attn_fp64(q[live], k8.float(), v8.float(), table[live], ll, scale, k_scale=ks, v_scale=vs)
+        _, l_deq = cf.attn_fp64(q[live], kd, vd, table[live], ll, scale)
+        torch.testing.assert_close(out[live].float(), ref_paged_attn(q[live], kd, vd, ll, table[live], scale).float(),
+                                   atol=OUT_ATOL, rtol=OUT_RTOL, msg=lambda m: f"{name} vs torch ref: {m}")
+        torch.testing.assert_close(out[live].double(), o64, atol=8e-3, rtol=1e-2, msg=lambda m: f"{name} vs exact cache: {m}")
+        torch.testing.assert_close(lse[live].double(), l64, atol=LSE_ATOL, rtol=0, msg=lambda m: f"{name} lse vs exact cache: {m}")
+        torch.testing.assert_close(lse[live].double(), l_deq, atol=5e-3, rtol=0, msg=lambda m: f"{name} lse vs dequantised: {m}")
+
+
 def test_what_is_not_built_for_two_segment_head_dims_is_refused(cuda_device):
     q, k, v, table, lens_t = _two_segment_inputs(cuda_device, (192, 128), [300, 20], (8, 2), 16, torch.bfloat16, 5)
     with pytest.raises(ValueError, match="matrix-core"):
         tda.flash_decode(q, k, v, table, lens_t, 1.0, algo="valu")
     with pytest.raises(ValueError, match="single-launch"):
         tda.prepare_decode(q, k, v, table, lens_t, 1.0, kv_split=4, single_launch=True).run()
-    k8, v8 = k.to(torch.float8_e4m3fn), v.to(torch.float8_e4m3fn)
-    with pytest.raises(ValueError, match="16-bit caches"):
-        tda.flash_decode(q, k8, v8, table, lens_t, 1.0)
     for dk, dv in ((192, 64), (128, 64), (576, 576), (256, 128)):
         qq = torch.zeros(2, 8, dk, dtype=torch.bfloat16, device=cuda_device)
         kk = torch.zeros(8, 16, 2, dk, dtype=torch.bfloat16, device=cuda_device)

@@ -10,9 +10,13 @@
     using RV = typename R::V;
     // K and V rows alike and of one power-of-two segment (head_dim 64, 128, 256): K and V loads pair up, every load
     // instruction covers the same rows, and all page modes, fp8 caches, two register buffers and the single-launch
-    // form are built.  Otherwise (192, 576 / 512 ...): 16-bit caches, one buffer, page numbers per tile or per row.
+    // form are built.  Otherwise (192, 576 / 512 ...): one buffer, page numbers per tile or per row.
     constexpr bool kOneSegment = DK == DV && RK::D1 == 0;
-    static_assert(kOneSegment || (!FP8 && NBUF == 1 && !PROBE && (PM == PM_TILE || PM == PM_ROW)), "not built");
+    // One-byte rows of 192 values are one and a half 128-byte lines: neighbouring kv heads of a token share a line, and
+    // workgroups with an odd number of kv heads are mapped so that those neighbours run on one XCD (one L2 fetches the
+    // line once; spread over the XCDs in dispatch order every head's L2 fetched both of its partial lines).
+    constexpr bool kRowsShareLines = !kOneSegment && FP8 && (DK % 128 != 0 || DV % 128 != 0);
+    static_assert(kOneSegment || (NBUF == 1 && !PROBE && (PM == PM_TILE || PM == PM_ROW)), "not built");
     static_assert(DK >= DV && DK % 32 == 0 && DV % 16 == 0, "K rows at least as long as V rows");
     constexpr int NJ = R::NJ;                  // (one segment)
     constexpr int LPR = R::LPR;                // lanes per cache row (one segment)
@@ -285,6 +289,45 @@
             for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int w = 0; w < 4; ++w) sink ^= rg.k[j][w] ^ rg.v[j][w];
+        } else if (FP8 && !kOneSegment) {
+            // rows of two segments: K and V have their own load instructions; 16 one-byte values become two 16-byte
+            // chunks of 16-bit values (chunk = value index / 8)
+            auto k_dequant = [&](const uint32_t (&in)[4], uint32_t (&o)[8]) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    if (fold) {
+                        o[2 * w] = P2::from_fp8(in[w], false);
+                        o[2 * w + 1] = P2::from_fp8(in[w], true);
+                    } else {
+                        const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(in[w], false);
+                        const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(in[w], true);
+                        o[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
+                        o[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
+                    }
+                }
+            };
+#pragma unroll
+            for (int j = 0; j < NJK; ++j) {
+                uint32_t ko[8];
+                k_dequant(rg.k[j], ko);
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+                    *reinterpret_cast<uint4*>(lds_k + k_off<RBK>(k_row(j), (k_byte(j) >> 3) + half)) =
+                        make_uint4(ko[4 * half], ko[4 * half + 1], ko[4 * half + 2], ko[4 * half + 3]);
+            }
+#pragma unroll
+            for (int j = 0; j < NJV; ++j) {
+                uint32_t vo[8];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    vo[2 * w] = P2::from_fp8(rg.v[j][w], false);
+                    vo[2 * w + 1] = P2::from_fp8(rg.v[j][w], true);
+                }
+#pragma unroll
+                for (int half = 0; half < 2; ++half)
+                    *reinterpret_cast<uint4*>(lds_v + v_off<RBV>(v_row(j), (v_byte(j) >> 3) + half)) =
+                        make_uint4(vo[4 * half], vo[4 * half + 1], vo[4 * half + 2], vo[4 * half + 3]);
+            }
         } else if (FP8) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
@@ -544,7 +587,7 @@
                 }
             }
         };
-        constexpr bool kSmallTiles = kTile * (DK + DV) * (FP8 ? 1 : 2) <= 4096;
+        constexpr bool kSmallTiles = kOneSegment ? kTile * (DK + DV) * (FP8 ? 1 : 2) <= 4096 : rows2_eight_share(FP8, DK, DV);
         if (ti_n == 1) merge(IntTag<1>());
         else if (ti_n == 2) merge(IntTag<2>());
         else if (ti_n == 4 || !kSmallTiles) merge(IntTag<4>());

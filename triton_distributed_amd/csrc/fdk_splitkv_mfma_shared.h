@@ -45,6 +45,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     static_assert(PM == PM_TILE || PM == PM_ROW, "page numbers per tile or per row");
     static_assert(DK % 64 == 0 && DV % 64 == 0, "the LDS swizzle acts on groups of eight 16-byte chunks");
     constexpr bool kOneSegment = false;        // (fdk_splitkv_mfma_work.h: several head tiles of a kv head go to one XCD)
+    constexpr bool kRowsShareLines = false;    // (16-bit rows: whole 128-byte lines per kv head)
     constexpr int kTileHeads = kSharedTileHeads;
     constexpr bool kFirstPieceStraight = false; // (fdk_splitkv_mfma_work.h: one copy of the piece, which needs every register)
     constexpr int NW = kSharedWaves;

@@ -38,6 +38,15 @@
                     ht = blockIdx.x % p.head_tiles;
                     hgb = blockIdx.x / p.head_tiles;
                 }
+            } else if (kRowsShareLines && (nh & 1) && p.hg_blocks > 1) {
+                // every unit of a (sequence, split) on one XCD: neighbouring kv heads share 128-byte lines
+                int row, unit;
+                tiles_on_one_xcd((int)(blockIdx.x + p.grid_x * (blockIdx.y + p.num_splits * blockIdx.z)),
+                                 p.num_splits * p.batch, p.grid_x, row, unit);
+                ht = unit % p.head_tiles;
+                hgb = unit / p.head_tiles;
+                split = row % p.num_splits;
+                pb = row / p.num_splits;
             } else if (p.head_tiles > 1) {
                 // the q-head tiles of a (sequence, split, kv-head block) on one XCD: see tiles_on_one_xcd
                 int row;
@@ -131,7 +140,9 @@
         int b = 0, before = 0, gb = 1;                // sequence of x, granules of the sequences before it, its granules
         int wc_of_wg = blockIdx.y, bu_of_wg = blockIdx.x;   // grid = (units, shares)
         if constexpr (!kOneSegment) {
-            if (p.head_tiles > 1) {                         // the q-head tiles of a (share, kv-head block) on one XCD
+            if (kRowsShareLines && (nh & 1) && p.hg_blocks > 1) {   // every unit of a share on one XCD
+                tiles_on_one_xcd((int)(blockIdx.x + p.grid_x * blockIdx.y), p.shares, p.grid_x, wc_of_wg, bu_of_wg);
+            } else if (p.head_tiles > 1) {                  // the q-head tiles of a (share, kv-head block) on one XCD
                 int row, tile;
                 tiles_on_one_xcd((int)(blockIdx.x + p.grid_x * blockIdx.y), p.hg_blocks * p.shares, p.head_tiles, row, tile);
                 bu_of_wg = (row % p.hg_blocks) * p.head_tiles + tile;

@@ -69,6 +69,11 @@ CONFIGS["d192v128_b32"] = DecodeConfig("d192v128_b32", 1302, 32, 32, 8, 192, 16,
                                        description="B32 32q/8kv Dk192 Dv128 N4096 P16 bf16")
 CONFIGS["d576v512_b32"] = DecodeConfig("d576v512_b32", 1303, 32, 128, 1, 576, 64, kv_len=4096, v_head_dim=512,
                                        description="B32 128q/1kv Dk576 Dv512 N4096 P64 bf16")
+CONFIGS["d192_fp8_b32"] = DecodeConfig("d192_fp8_b32", 1304, 32, 32, 8, 192, 16, kv_len=4096, kv_dtype="fp8_e4m3",
+                                       description="B32 32q/8kv Dk192 Dv192 N4096 P16, e4m3 KV with per-kv-head scales")
+CONFIGS["d576v512_fp8_b32"] = DecodeConfig("d576v512_fp8_b32", 1305, 32, 128, 1, 576, 64, kv_len=4096, v_head_dim=512,
+                                           kv_dtype="fp8_e4m3",
+                                           description="B32 128q/1kv Dk576 Dv512 N4096 P64, e4m3 KV with per-kv-head scales")
 
 # The shape behind the reference's only published figure for this path (README.md:200-202; perf loops of
 # test/nvidia/test_sp_decode_attn.py:203-220 and test_decode_attn.py:294-527): batch 1, 96 q / 12 kv heads,
