@@ -435,29 +435,31 @@ def test_large_groups_on_one_kv_head_share_the_staged_tiles(cuda_device, heads, 
 
 
 @pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
-@pytest.mark.parametrize("heads,page", [((32, 8), 16), ((16, 2), 4), ((40, 1), 64), ((128, 1), 16)])
+@pytest.mark.parametrize("heads,page", [((32, 8), 16), ((16, 2), 4), ((40, 1), 64), ((128, 1), 16), ((66, 2), 6), ((128, 2), 1)])
 def test_two_segment_head_dims_with_an_fp8_cache(cuda_device, dims, heads, page):
     """e4m3 caches with per-kv-head scales behind rows of two segments: exact dequantisation (the decode over the
-    dequantised cache) and the K scale folded into the logit scale, through a single pass, chunks and equal shares; large
-    groups run with tiles of 16 q heads here."""
+    dequantised cache) and the K scale folded into the logit scale, through a single pass, chunks, a work queue and equal
+    shares; groups of more than 32 q heads on rows of 576 / 512 values run in the kernels that share the staged tiles.
+    fp16 queries at page size 6."""
     dk, dv = dims
     hq, hkv = heads
     g = torch.Generator().manual_seed(dk + hq + page)
     lens = [int(x) for x in torch.randint(1, 1800, (5,), generator=g)]
     lens[1] = 0
-    q, k16, v16, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, heads, page, torch.bfloat16, 900 + hq + page)
+    dtype = torch.float16 if page == 6 else torch.bfloat16
+    q, k16, v16, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, heads, page, dtype, 900 + hq + page)
     k16[-1], v16[-1] = 0, 0                          # (the page of NaN does not quantise)
     k8, ks = wl.quantize_kv_fp8(k16)
     v8, vs = wl.quantize_kv_fp8(v16)
     k8.view(torch.uint8)[-1] = 0x7F                  # unused table columns still point at NaN (0x7F in e4m3)
     v8.view(torch.uint8)[-1] = 0x7F
-    kd, vd = ofp8.dequant_per_head(k8, ks), ofp8.dequant_per_head(v8, vs)
+    kd, vd = ofp8.dequant_per_head(k8, ks, dtype), ofp8.dequant_per_head(v8, vs, dtype)
     scale = dk ** -0.5
     live = [i for i, n in enumerate(lens) if n > 0]
     plan = tda.get_split_kv_plan(q, k8, v8, table, lens_t, scale)
     assert plan.algo == "mfma"
-    for tag, kw in (("auto", {}), ("single pass", dict(kv_split=1)), ("3 chunks", dict(kv_split=3)), ("equal shares", dict(force_balanced=True)),
-                    ("folded", dict(fp8_fold_k_scale=True))):
+    for tag, kw in (("auto", {}), ("single pass", dict(kv_split=1)), ("3 chunks", dict(kv_split=3)), ("queue", dict(kv_split=40)),
+                    ("equal shares", dict(force_balanced=True)), ("folded", dict(fp8_fold_k_scale=True))):
         out, lse = tda.flash_decode(q, k8, v8, table, lens_t, scale, k_scale=ks, v_scale=vs, **kw)
         torch.cuda.synchronize()
         assert out.shape == (len(lens), hq, dv)

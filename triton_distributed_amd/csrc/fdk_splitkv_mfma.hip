@@ -40,8 +40,8 @@ bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim, int 
 // q heads of one kv head that a workgroup covers: a tile of 16 (a wavefront per kv head), or 64 where the rows are
 // long and the group is large - latent attention, 128 q heads on one kv head of 576 + 512 values - and the kernels of
 // fdk_splitkv_mfma_shared.h load and stage every tile once for four tiles of 16 q heads
-int mfma_heads_per_wg(int group, int row_values, int kv_dtype) {
-    return row_values > 512 && group > 32 && kv_dtype != FDK_FP8_E4M3 ? 64 : 16;
+int mfma_heads_per_wg(int group, int row_values) {
+    return row_values > 512 && group > 32 ? 64 : 16;
 }
 
 // kv heads per workgroup.  Adjacent kv heads of a token are adjacent in the cache, so a workgroup that takes
@@ -55,8 +55,8 @@ int mfma_heads_per_wg(int group, int row_values, int kv_dtype) {
 // the number of independent workgroups.
 // (Rows of more than 512 values per token and kv head, K and V together: at most two heads, i.e. the four wavefronts
 // that the registers and the LDS of a compute unit hold at that size.)
-int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values, int kv_dtype) {
-    if (mfma_heads_per_wg(group, row_values, kv_dtype) > 16) return 1;   // the shared-tile kernels: one kv head, 64 q heads
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values) {
+    if (mfma_heads_per_wg(group, row_values) > 16) return 1;   // the shared-tile kernels: one kv head, 64 q heads
     const int head_tiles = (group + 15) / 16;
     for (int nh = row_values > 512 ? 2 : 8; nh >= 1; nh >>= 1) {
         if (hkv % nh) continue;

@@ -18,7 +18,7 @@
 // kernels (fdk_splitkv_mfma_body.h): S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with
 // 16x16x16 MFMA and P rounded to the cache dtype; the QK product runs as six interleaved accumulation chains (18
 // dependent MFMA would wait for each other), and the running maximum of the softmax is a reference that moves rarely,
-// so that the tile loop holds no rescale of the output tile (see move_reference).  16-bit caches; page numbers per tile
+// so that the tile loop holds no rescale of the output tile (see move_reference).  16-bit and e4m3 caches; page numbers per tile
 // or per row (PM_TILE, PM_ROW).  How pieces are handed out is shared with the other kernels
 // (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
 #pragma once
@@ -36,12 +36,13 @@ constexpr int kSharedTileHeads = 16 * kSharedWaves / kSharedColSplit;    // q he
 
 // REUSE: another workgroup reads the same K / V rows (a group of more than 64 q heads): plain loads, so that the rows
 // stay in the XCD's L2 for it; otherwise the rows are read once and come with the non-temporal hint.
-template <int QDT, int PM, int DK, int DV, int MODE, bool REUSE>
+// FP8: an e4m3 cache; the rows are dequantised on their way into the staged tile, which holds 16-bit values either way.
+template <int QDT, int PM, int DK, int DV, int MODE, bool REUSE, bool FP8 = false>
 __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(const SplitParams p) {
     using M = Mma<QDT>;
     using P2 = Pack2<QDT>;
-    using RK = Rows<false, DK>;
-    using RV = Rows<false, DV>;
+    using RK = Rows<FP8, DK>;
+    using RV = Rows<FP8, DV>;
     static_assert(PM == PM_TILE || PM == PM_ROW, "page numbers per tile or per row");
     static_assert(DK % 64 == 0 && DV % 64 == 0, "the LDS swizzle acts on groups of eight 16-byte chunks");
     constexpr bool kOneSegment = false;        // (fdk_splitkv_mfma_work.h: several head tiles of a kv head go to one XCD)
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr int kTileHeads = kSharedTileHeads;
     constexpr bool kFirstPieceStraight = false; // (fdk_splitkv_mfma_work.h: one copy of the piece, which needs every register)
     constexpr int NW = kSharedWaves;
-    constexpr int ES = 2;
+    constexpr int ES = FP8 ? 1 : 2;            // bytes per cache value
     constexpr int RBK = 2 * DK, RBV = 2 * DV;  // bytes of a staged row
     constexpr int KS = DK / 32;                // k-steps of the QK product
     constexpr int CS = kSharedColSplit;
@@ -126,6 +127,17 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
 
         const bool softcap = p.soft_cap > 0.f;
         const float inv_cap = softcap ? 1.0f / p.soft_cap : 0.f;
+        // e4m3 caches, as in the other kernels: K becomes (k8 * k_scale) rounded to the q dtype on its way into LDS - the
+        // dequantised cache that the reference would decode - or, folded, the exact k8 with k_scale in the logit scale;
+        // V is converted exactly and v_scale multiplies the output rows once at the end
+        float kscale = 1.f, vscale = 1.f;
+        if (FP8) {
+            if (p.k_scale) kscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.k_scale))[kvh]);
+            if (p.v_scale) vscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.v_scale))[kvh]);
+        }
+        const bool fold = FP8 && p.fp8_fold;
+        const float logit_scale_log2 = fold ? p.scale_log2 * kscale : p.scale_log2;
+        const float logit_scale = fold ? p.sm_scale * kscale : p.sm_scale;
         const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;
         const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
         const uint32_t ksp_bytes = (uint32_t)(p.k_sp * ES), vsp_bytes = (uint32_t)(p.v_sp * ES);
@@ -202,7 +214,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             }
         };
         // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
-        // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
         auto stage = [&](const Tile& rg, char* buf) {
             char* lk = buf;
             char* lv = buf + kTile * RBK;
@@ -212,27 +223,67 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             int ln = lane;
             asm volatile("" : "+v"(ln));
             ln &= 63;                                       // (known to the compiler again: a row of 64 lanes is one row)
+            // one register quadruple to its place in a staged row: 16 bytes of a 16-bit cache are one chunk; 16 one-byte
+            // values become two chunks of 16-bit values
+            auto store_k = [&](const uint32_t (&r)[4], int row, int piece) {
+                if constexpr (!FP8) {
+                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(row, piece)) = get(r);
+                } else {
+                    uint32_t o[8];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        if (fold) {
+                            o[2 * w] = P2::from_fp8(r[w], false);
+                            o[2 * w + 1] = P2::from_fp8(r[w], true);
+                        } else {
+                            const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], false);
+                            const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], true);
+                            o[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
+                            o[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
+                        }
+                    }
+#pragma unroll
+                    for (int half = 0; half < 2; ++half)
+                        *reinterpret_cast<uint4*>(lk + k_off<RBK>(row, 2 * piece + half)) =
+                            make_uint4(o[4 * half], o[4 * half + 1], o[4 * half + 2], o[4 * half + 3]);
+                }
+            };
+            auto store_v = [&](const uint32_t (&r)[4], int row, int piece) {
+                if constexpr (!FP8) {
+                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, piece)) = get(r);
+                } else {
+                    uint32_t o[8];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        o[2 * w] = P2::from_fp8(r[w], false);
+                        o[2 * w + 1] = P2::from_fp8(r[w], true);
+                    }
+#pragma unroll
+                    for (int half = 0; half < 2; ++half)
+                        *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, 2 * piece + half)) =
+                            make_uint4(o[4 * half], o[4 * half + 1], o[4 * half + 2], o[4 * half + 3]);
+                }
+            };
+            // (piece: the lane's 16 bytes within the cache row, counted in 16-byte pieces)
 #pragma unroll
             for (int s = 0; s < KS0; ++s) {
                 const int j = slot_instr(s, RK::NJ0);
-                *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0)) = get(rg.k[s]);
+                store_k(rg.k[s], j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0);
             }
 #pragma unroll
             for (int s = 0; s < KS1; ++s) {
                 const int j = slot_instr(s, RK::NJ1);
-                *reinterpret_cast<uint4*>(lk + k_off<RBK>(j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1)) =
-                    get(rg.k[KS0 + s]);
+                store_k(rg.k[KS0 + s], j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1);
             }
 #pragma unroll
             for (int s = 0; s < VS0; ++s) {
                 const int j = slot_instr(s, RV::NJ0);
-                *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0)) = get(rg.v[s]);
+                store_v(rg.v[s], j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0);
             }
 #pragma unroll
             for (int s = 0; s < VS1; ++s) {
                 const int j = slot_instr(s, RV::NJ1);
-                *reinterpret_cast<uint4*>(lv + v_off<RBV>(j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1)) =
-                    get(rg.v[VS0 + s]);
+                store_v(rg.v[VS0 + s], j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1);
             }
         };
 
@@ -314,10 +365,10 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             float sv[4] = {s.x, s.y, s.z, s.w};
             if (softcap) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * p.sm_scale, p.soft_cap, inv_cap) * kLog2e;
+                for (int i = 0; i < 4; ++i) sv[i] = soft_cap_fn(sv[i] * logit_scale, p.soft_cap, inv_cap) * kLog2e;
             } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sv[i] *= p.scale_log2;
+                for (int i = 0; i < 4; ++i) sv[i] *= logit_scale_log2;
             }
             if (MASKED) {                         // the last tile of the piece may be partial
 #pragma unroll
@@ -415,7 +466,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         l_run += __shfl_xor(l_run, 32, 64);
         if (c < heads_here) {
             const int hq = head0 + c;
-            const float norm = fast_rcp(l_run);                     // > 0: the piece holds a token
+            const float norm = FP8 ? vscale * fast_rcp(l_run) : fast_rcp(l_run);   // l_run > 0: the piece holds a token
             const float lse_nat = (m_ref + fast_log2(l_run)) * kLn2;
             const int64_t prow = prow0 + (int64_t)(16 * wtile + c) * prow_step;
 #pragma unroll
@@ -440,8 +491,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
 }
 
 // Launch of the shared-tile kernels.  The plan counts head tiles of kSharedTileHeads q heads and one kv head per
-// workgroup for them (mfma_tile_heads, mfma_kv_heads_per_wg).
-template <int QDT, int DK, int DV, int MODE>
+// workgroup for them (mfma_heads_per_wg, mfma_kv_heads_per_wg).
+template <int QDT, int DK, int DV, int MODE, bool FP8>
 int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     if (mfma_work_mode(p_in) != MODE || p_in.fused || p_in.probe || p_in.hg_per_wg != 1 || p_in.tile_heads != kSharedTileHeads)
         return (int)hipErrorInvalidValue;
@@ -469,10 +520,10 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
 #define FDK_SHARED_LAUNCH(PMV, RU)                                                                                        \
     do {                                                                                                                  \
         const hipError_t e = hipFuncSetAttribute(                                                                         \
-            reinterpret_cast<const void*>(&splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU>),                       \
+            reinterpret_cast<const void*>(&splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU, FP8>),                  \
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);                                                  \
         if (e != hipSuccess) return (int)e;                                                                               \
-        hipLaunchKernelGGL((splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU>), grid, block, lds_bytes, stream, p);  \
+        hipLaunchKernelGGL((splitkv_mfma_shared_kernel<QDT, PMV, DK, DV, MODE, RU, FP8>), grid, block, lds_bytes, stream, p); \
     } while (0)
     if (pm == PM_TILE) {
         if (reuse) FDK_SHARED_LAUNCH(PM_TILE, true);
@@ -487,8 +538,10 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
 
 template <int DK, int DV, int MODE>
 int launch_mfma_shared(const SplitParams& p, int q_dtype, int kv_dtype, hipStream_t stream) {
+    if (kv_dtype == FDK_FP8_E4M3)
+        return q_dtype == FDK_BF16 ? launch_shared<FDK_BF16, DK, DV, MODE, true>(p, stream) : launch_shared<FDK_FP16, DK, DV, MODE, true>(p, stream);
     if (kv_dtype != q_dtype) return (int)hipErrorInvalidValue;
-    return q_dtype == FDK_BF16 ? launch_shared<FDK_BF16, DK, DV, MODE>(p, stream) : launch_shared<FDK_FP16, DK, DV, MODE>(p, stream);
+    return q_dtype == FDK_BF16 ? launch_shared<FDK_BF16, DK, DV, MODE, false>(p, stream) : launch_shared<FDK_FP16, DK, DV, MODE, false>(p, stream);
 }
 
 }  // namespace
