@@ -434,6 +434,51 @@ def test_large_groups_on_one_kv_head_share_the_staged_tiles(cuda_device, heads, 
     torch.testing.assert_close(packed[live][..., 512].float(), lse_a[live], atol=3e-2, rtol=1e-2)
 
 
+def _quantized_two_segment(k16, v16, dtype):
+    """e4m3 caches with per-kv-head scales from the 16-bit caches of _two_segment_inputs (whose last page holds NaN for
+    the unused table columns), and what they dequantise to in ``dtype``."""
+    k16[-1], v16[-1] = 0, 0                          # (the page of NaN does not quantise)
+    k8, ks = wl.quantize_kv_fp8(k16)
+    v8, vs = wl.quantize_kv_fp8(v16)
+    k8.view(torch.uint8)[-1] = 0x7F                  # unused table columns still point at NaN (0x7F in e4m3)
+    v8.view(torch.uint8)[-1] = 0x7F
+    return k8, ks, v8, vs, ofp8.dequant_per_head(k8, ks, dtype), ofp8.dequant_per_head(v8, vs, dtype)
+
+
+@pytest.mark.parametrize("seed", list(range(24)))
+def test_two_segment_head_dims_random_shapes_with_an_fp8_cache(cuda_device, seed):
+    g = torch.Generator().manual_seed(7000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    dims = TWO_SEGMENT_DIMS[seed % 3]
+    hkv = [1, 2, 3, 4, 8][r(0, 4)]
+    group = [1, 2, 4, 7, 8, 16, 20, 40, 64, 100, 128][r(0, 10)]
+    page = [1, 2, 5, 8, 16, 32, 48, 128][r(0, 7)]
+    batch = r(1, 16)
+    top = [60, 700, 4000][r(0, 2)]
+    lens = [r(0 if batch > 1 else 1, top) for _ in range(batch)]
+    if max(lens) == 0:
+        lens[0] = 17
+    dtype = [torch.bfloat16, torch.float16][r(0, 1)]
+    cap = [0.0, 20.0][r(0, 1)]
+    split = [-1, -1, 1, 2, 7, 33][r(0, 5)]
+    hints = r(0, 1)
+    print(f"case fp8 seed={seed} dims={dims} heads=({hkv * group},{hkv}) P={page} B={batch} top={top} {dtype} cap={cap} "
+          f"split={split} hints={hints}", flush=True)
+    q, k16, v16, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, (hkv * group, hkv), page, dtype, 8000 + seed,
+                                                     table_extra=r(0, 3))
+    k8, ks, v8, vs, kd, vd = _quantized_two_segment(k16, v16, dtype)
+    scale = dims[0] ** -0.5
+    kw = dict(max_kv_len=max(lens), min_kv_len=min(lens)) if hints else {}
+    out, lse = tda.flash_decode(q, k8, v8, table, lens_t, scale, soft_cap=cap, kv_split=split, k_scale=ks, v_scale=vs, **kw)
+    torch.cuda.synchronize()
+    live = [i for i, n in enumerate(lens) if n > 0]
+    for i, n in enumerate(lens):
+        if n == 0:
+            assert float(out[i].abs().max()) == 0 and bool((lse[i] == -math.inf).all())
+    _check(out[live], lse[live], q[live], k8, v8, table[live], [lens[i] for i in live], scale, cap, ref_kv=(kd, vd),
+           tag=f"fp8 seed {seed}")
+
+
 @pytest.mark.parametrize("dims", TWO_SEGMENT_DIMS)
 @pytest.mark.parametrize("heads,page", [((32, 8), 16), ((16, 2), 4), ((40, 1), 64), ((128, 1), 16), ((66, 2), 6), ((128, 2), 1)])
 def test_two_segment_head_dims_with_an_fp8_cache(cuda_device, dims, heads, page):
@@ -448,12 +493,7 @@ def test_two_segment_head_dims_with_an_fp8_cache(cuda_device, dims, heads, page)
     lens[1] = 0
     dtype = torch.float16 if page == 6 else torch.bfloat16
     q, k16, v16, table, lens_t = _two_segment_inputs(cuda_device, dims, lens, heads, page, dtype, 900 + hq + page)
-    k16[-1], v16[-1] = 0, 0                          # (the page of NaN does not quantise)
-    k8, ks = wl.quantize_kv_fp8(k16)
-    v8, vs = wl.quantize_kv_fp8(v16)
-    k8.view(torch.uint8)[-1] = 0x7F                  # unused table columns still point at NaN (0x7F in e4m3)
-    v8.view(torch.uint8)[-1] = 0x7F
-    kd, vd = ofp8.dequant_per_head(k8, ks, dtype), ofp8.dequant_per_head(v8, vs, dtype)
+    k8, ks, v8, vs, kd, vd = _quantized_two_segment(k16, v16, dtype)
     scale = dk ** -0.5
     live = [i for i, n in enumerate(lens) if n > 0]
     plan = tda.get_split_kv_plan(q, k8, v8, table, lens_t, scale)
