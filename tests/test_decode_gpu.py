@@ -353,17 +353,22 @@ def test_two_segment_head_dims_random_shapes(cuda_device, seed):
            ref_tol=4e-2 if scale > dims[0] ** -0.5 else None)
 
 
-@pytest.mark.parametrize("dims,heads", [(d, (32, 2)) for d in TWO_SEGMENT_DIMS] + [((576, 512), (128, 1))])
-def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(cuda_device, dims, heads):
+@pytest.mark.parametrize("dims,heads,fp8", [(d, (32, 2), False) for d in TWO_SEGMENT_DIMS] + [((576, 512), (128, 1), False),
+                                                     ((192, 192), (24, 3), True), ((576, 512), (128, 1), True)])
+def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(cuda_device, dims, heads, fp8):
     """A captured call (the kernels of the widest rows ask for more LDS than the default limit at launch; 128 q heads on one
     kv head: the kernels whose wavefronts share the staged tiles) replayed on changed q and lengths, and the entry point
-    that allocates nothing, against the eager call."""
+    that allocates nothing, against the eager call.  16-bit and e4m3 caches."""
     dk, dv = dims
     g = torch.Generator().manual_seed(dk * 3 + dv)
     q, k, v, table, lens_t = _two_segment_inputs(cuda_device, dims, [2500] * 4, heads, 16, torch.bfloat16, 31)   # pages for every length below
+    ref_kv, kw8 = None, {}
+    if fp8:
+        k, ks, v, vs, kd, vd = _quantized_two_segment(k, v, torch.bfloat16)
+        ref_kv, kw8 = (kd, vd), dict(k_scale=ks, v_scale=vs)
     lens_t.copy_(_lens_t([2500, 1, 900, 1800], cuda_device))
     scale = dk ** -0.5
-    call = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500)
+    call = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500, **kw8)
     assert call.plan.num_splits > 1
     call.run()
     torch.cuda.synchronize()
@@ -378,8 +383,8 @@ def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(
         graph.replay()
         torch.cuda.synchronize()
         got_o, got_l = call.out.clone(), call.lse.clone()
-        want_o, want_l = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=2500)
-        static = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500, static_scratch=True)
+        want_o, want_l = tda.flash_decode(q, k, v, table, lens_t, scale, max_kv_len=2500, **kw8)
+        static = tda.prepare_decode(q, k, v, table, lens_t, scale, max_kv_len=2500, static_scratch=True, **kw8)
         if call.plan.workspace_bytes <= 32 << 20:
             st_o, st_l = static.run_static()
         else:                                   # (128 q heads x 32 splits x 512 values: beyond the 32 MiB the library holds)
@@ -390,8 +395,8 @@ def test_two_segment_head_dims_under_graph_capture_and_through_the_static_entry(
         assert torch.equal(got_o, want_o) and torch.equal(got_l, want_l), f"replay {i}"
         assert torch.equal(st_o, want_o) and torch.equal(st_l, want_l), f"static entry {i}"
         live = [j for j, n in enumerate(new_lens) if n > 0]
-        _check(got_o[live], got_l[live], q[live], k, v, table[live], [new_lens[j] for j in live], scale,
-               tag=f"dims={dims} graph replay {i}")
+        _check(got_o[live], got_l[live], q[live], k, v, table[live], [new_lens[j] for j in live], scale, ref_kv=ref_kv,
+               tag=f"dims={dims} fp8={fp8} graph replay {i}")
 
 
 @pytest.mark.parametrize("heads", [(128, 1), (128, 2), (64, 1), (40, 1), (66, 2)])

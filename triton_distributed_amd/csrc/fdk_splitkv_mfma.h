@@ -426,7 +426,7 @@ int launch_rows2(const SplitParams& p_in, hipStream_t stream) {
     // rows of 192 values, an odd number of kv heads per workgroup; measured, batch 32 x 8 kv heads x 4096 tokens in a single
     // pass: 88.3 -> 72.9 us, memory traffic 1.29 -> 1.00 of the bytes attended to; with two heads per workgroup plain loads
     // are 3 % slower than streaming ones)
-    const bool reuse = p.head_tiles > 1 || (FP8 && (DK % 128 != 0 || DV % 128 != 0) && (p.hg_per_wg & 1));
+    const bool reuse = p.head_tiles > 1 || (FP8 && (DK % 128 != 0 || DV % 128 != 0) && (p.hg_per_wg & 1) && p.hg_blocks > 1);
 #define FDK_ROWS2_LAUNCH(PMV, RU)                                                                                          \
     do {                                                                                                                   \
         if (lds_bytes > 64 * 1024) {                                                                                       \
