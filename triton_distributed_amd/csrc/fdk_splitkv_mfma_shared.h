@@ -56,6 +56,19 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr int CS = kSharedColSplit;
     constexpr int DB = DV / 16 / CS;           // 16-column blocks of the output that this wavefront holds
     constexpr int kTileBytes = kTile * (RBK + RBV);
+    // 16-bit caches: the rows go from memory straight into the staged tile (global_load_lds_dwordx4: lane i of a load
+    // instruction writes its 16 bytes at M0 + 16 i, no registers in between and nothing to store), three staged tiles.
+    // A load instruction then fills 1 KB of consecutive LDS, so the second K segment of the 16 rows lies behind their
+    // first segments instead of behind each row, and the swizzle is applied on the memory side: the lane whose bytes
+    // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).  e4m3 caches pass
+    // through registers for the conversion (two staged tiles).
+    constexpr bool kDirect = !FP8;
+    constexpr int kStaged = kDirect ? 3 : 2;   // staged tiles in LDS
+    static_assert(!kDirect || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
+                  "direct loads: a first segment of 1 KB per row, a second K segment of 128 bytes");
+    constexpr int kK0Row = kDirect ? RK::D0 * 2 : RBK;                 // bytes from one staged row's first K segment to the next row's
+    constexpr int kK1Base = kDirect ? kTile * RK::D0 * 2 : RK::D0 * 2; // where row 0's second K segment starts, and
+    constexpr int kK1Row = kDirect ? RK::D1 * 2 : RBK;                 // the step to the next row's
     // load instructions of a tile that one wavefront issues, per segment of the rows (Rows<>)
     constexpr int KS0 = (RK::NJ0 + NW - 1) / NW, KS1 = (RK::NJ1 + NW - 1) / NW;
     constexpr int VS0 = (RV::NJ0 + NW - 1) / NW, VS1 = (RV::NJ1 + NW - 1) / NW;
@@ -69,7 +82,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     const int nh = 1, hl = 0, tix = 0;         // one kv head per workgroup; every wavefront sees every tile
     const int wtile = wave / CS;               // this wavefront's tile of 16 q heads within the workgroup's
     const int whalf = wave % CS;               // ... and its part of the output columns
-    int* const s_next = reinterpret_cast<int*>(lds + 2 * kTileBytes);
+    int* const s_next = reinterpret_cast<int*>(lds + kStaged * kTileBytes);
 
     auto write_empty_rows = [&](const int b, const int head0, const int heads_here) {
         for (int idx = lane; idx < heads_here * DV; idx += 64) {
@@ -102,12 +115,15 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         uint4 qreg[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qreg[ks] = make_uint4(0, 0, 0, 0);
-        if (active) {
-            const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
-                                 (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
+        auto load_q = [&]() {
+            if (active) {
+                const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
+                                     (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
-        }
+                for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+            }
+        };
+        if (!kDirect) load_q();                 // (direct loads: requested behind the first rows, see the tile loop)
         const ConstI32 tbl = as_const(p.block_table + (int64_t)b * p.tbl_sb);
         const int pmask = p.page_size - 1;
         const int kv_len = min(as_const(p.kv_lens)[b], p.max_tokens);
@@ -169,19 +185,60 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             const int j = NW * s + wave;
             return j < n ? j : j % n;
         };
-        auto load_rows = [&](auto clamp_tag, int tok0, int32_t pg_id, int first_row, int lane_row, uint32_t lane_off,
-                             uint32_t lane_byte, const char* plane, uint32_t sp_bytes, uint32_t st_bytes) {
+        auto row_ptr = [&](auto clamp_tag, int tok0, int32_t pg_id, int first_row, int lane_row, uint32_t lane_off,
+                           uint32_t lane_byte, const char* plane, uint32_t sp_bytes, uint32_t st_bytes) {
             constexpr bool CLAMP = decltype(clamp_tag)::value;
             if (PM == PM_TILE && !CLAMP) {
                 // the tile lies in one page: a wave-uniform base plus the lane's offset
                 const int n0 = tok0 + first_row;
-                return load16(plane + ((uint64_t)(uint32_t)pg_id * sp_bytes + (uint64_t)((uint32_t)(n0 & pmask) * st_bytes)) + lane_off);
+                return plane + ((uint64_t)(uint32_t)pg_id * sp_bytes + (uint64_t)((uint32_t)(n0 & pmask) * st_bytes)) + lane_off;
             }
             int n = tok0 + first_row + lane_row;
             if (CLAMP) n = min(n, c_end - 1);
             const uint32_t slot = PM == PM_TILE ? (uint32_t)(n & pmask) : (uint32_t)(p.page_shift < 0 ? n % p.page_size : (n & pmask));
             const uint32_t pg = (uint32_t)(PM == PM_TILE ? pg_id : __shfl(pg_id, n - tok0, 64));
-            return load16(plane + ((uint64_t)pg * sp_bytes + (uint64_t)(slot * st_bytes)) + lane_byte);
+            return plane + ((uint64_t)pg * sp_bytes + (uint64_t)(slot * st_bytes)) + lane_byte;
+        };
+        auto load_rows = [&](auto clamp_tag, int tok0, int32_t pg_id, int first_row, int lane_row, uint32_t lane_off,
+                             uint32_t lane_byte, const char* plane, uint32_t sp_bytes, uint32_t st_bytes) {
+            return load16(row_ptr(clamp_tag, tok0, pg_id, first_row, lane_row, lane_off, lane_byte, plane, sp_bytes, st_bytes));
+        };
+        // ---- direct loads (kDirect): 16 bytes per lane from memory to LDS byte (dst + 16 lane), dst wave-uniform.  The
+        // compiler does not see these loads (it would wait for ALL loads under way in front of every LDS read that follows
+        // one): the tile loop places its own waits, see there. ----
+        auto load_to_lds16 = [&](const char* ptr, uint32_t dst) {
+            if (REUSE) asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(ptr), "s"(dst) : "memory");
+            else asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(ptr), "s"(dst) : "memory");
+        };
+        constexpr int kLoadsPerTile = KS0 + KS1 + VS0 + VS1;        // load instructions of a tile that a wavefront issues
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) char*)lds;    // the LDS byte address of lds[0]
+        // Tile t into the staged tile at LDS byte dst.  A lane fetches the chunk that the swizzle of the staged tile
+        // (k_off, v_off) wants where its bytes land: first segments, one row per instruction: chunk lane ^ swizzle(row);
+        // second K segment, eight rows of eight chunks per instruction: chunk (lane & 7) ^ (row & 7) of row lane >> 3.
+        auto issue_direct = [&](auto clamp_tag, int t, int32_t pg_id, uint32_t dst) {
+            const int tok0 = c_start + t * kTile;
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            ln &= 63;
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                const uint32_t byte = (uint32_t)((ln ^ (j & 7)) << 4);
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j, 0, byte, byte, kplane, ksp_bytes, kst_bytes), dst + j * 1024);
+            }
+#pragma unroll
+            for (int s = 0; s < KS1; ++s) {
+                const int j = slot_instr(s, RK::NJ1);
+                const uint32_t byte = (uint32_t)(RK::D0 * ES + (((ln & 7) ^ ((ln >> 3) & 7)) << 4));
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j * 8, ln >> 3, (uint32_t)(ln >> 3) * kst_bytes + byte, byte, kplane,
+                                      ksp_bytes, kst_bytes), dst + kK1Base + j * 1024);
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                const uint32_t byte = (uint32_t)((ln ^ ((j & 3) << 1)) << 4);
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j, 0, byte, byte, vplane, vsp_bytes, vst_bytes), dst + kTile * RBK + j * 1024);
+            }
         };
         auto issue = [&](auto clamp_tag, int t, int32_t pg_id, Tile& rg) {
             const int tok0 = c_start + t * kTile;
@@ -328,8 +385,12 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             //   K operand of k-step ks: row c, chunk 4 ks + a  ->  chunk ^ (c & 7) = 8 (ks >> 1) + ((4 (ks & 1) + a) ^ (c & 7))
             //   V operand of block db (transposed read): row 4 a + (c >> 2), chunk 2 db + ((c & 3) >> 1)
             //                                            ->  2 (4 (db >> 2) + ((db & 3) ^ (row & 3))) + ((c & 3) >> 1)
-            const char* lk = buf + c * RBK;
+            const char* lk = buf + c * kK0Row;
             const char* k_at[2] = {lk + (((0 + a) ^ (c & 7)) << 4), lk + (((4 + a) ^ (c & 7)) << 4)};
+            // (k-steps of the second K segment: from row c's second segment on, which in the direct-load layout lies
+            // elsewhere than behind its first)
+            constexpr int KSEG0 = RK::D0 / 32;
+            const int k1_delta = kK1Base + c * (kK1Row - kK0Row) - KSEG0 / 2 * 128;
             const int k4 = c >> 2, cc = c & 3;
             const int vrow = 4 * a + k4;
             const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8 + whalf * (DB / 4) * 128;   // (+ this wavefront's columns)
@@ -348,7 +409,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
 #pragma unroll
                 for (int i = 0; i < QG; ++i) {
                     const int ks = g * QG + i;
-                    ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + (ks >> 1) * 128);
+                    if (kDirect && ks >= KSEG0) ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + k1_delta + (ks >> 1) * 128);
+                    else ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + (ks >> 1) * 128);
                 }
             };
             read_qk(0, 0);
@@ -414,7 +476,62 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // in order, so waiting for a number then never waits for rows requested after it.
         // (A wavefront that leaves the inner loop to move its reference does so after the tile's barrier and comes back for
         // the next tile: every wavefront passes exactly one barrier per tile.) ----
-        {
+        if constexpr (kDirect) {
+            // Direct loads, three staged tiles: tile t is read from buffer t % 3 while the loads of tiles t + 1 and t + 2 are
+            // under way into the other two.  Per tile: wait until this wavefront's loads of tile t have landed, barrier
+            // (every wavefront's have, and every wavefront has finished with tile t - 1), request tile t + 2 into the buffer
+            // of tile t - 1, work on tile t.  Every wavefront issues exactly kLoadsPerTile loads per tile, and loads return
+            // in order: "tile t has landed" is "at most kLoadsPerTile loads under way" while tile t + 1 has been requested,
+            // "none under way" for the last tile.  (Loads that the compiler sees - page numbers per row, PM_ROW - only make
+            // these waits, and the compiler's own, wait for more than they need.)
+            const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
+            auto issue_tile = [&](int t, int32_t pg_id) {
+                const uint32_t dst = lds0 + (uint32_t)(t % 3) * kTileBytes;
+                if (t < n_full) issue_direct(BoolTag<false>(), t, pg_id, dst);
+                else if (t < n_tiles) issue_direct(BoolTag<true>(), t, pg_id, dst);
+            };
+            // the staged tiles are free: no wavefront still reads the previous piece's, none of its loads is under way
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            int32_t pg_a = page_id(2), pg_b = page_id(3);           // (a: even tiles, b: odd tiles)
+            issue_tile(0, page_id(0));
+            issue_tile(1, page_id(1));
+            load_q();
+            // Q^T has to have arrived HERE: the compiler would otherwise wait for its loads where they are first used, inside
+            // the tile loop, by counting down to "no load under way" - in every iteration, and the rows requested for the
+            // tiles ahead are loads it does not know of.  (An empty asm that takes the registers as operands is such a use.)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
+            auto land_and_issue = [&](int t, int32_t& pg) {
+                static_assert(kLoadsPerTile == 5, "the wait below counts the loads of one tile");
+                if (t + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+                const int32_t pg_now = pg;
+                pg = page_id(t + 4);
+                issue_tile(t + 2, pg_now);
+            };
+            int t = 0;
+            for (;;) {
+                bool gave_up = false;
+                for (; t < n_full; ++t) {
+                    if (t & 1) land_and_issue(t, pg_b);
+                    else land_and_issue(t, pg_a);
+                    if (active && !try_compute(t, lds + (t % 3) * kTileBytes, BoolTag<false>())) {
+                        gave_up = true;
+                        break;
+                    }
+                }
+                if (!gave_up) break;
+                do move_reference(); while (!try_compute(t, lds + (t % 3) * kTileBytes, BoolTag<false>()));
+                ++t;
+            }
+            if (n_full < n_tiles) {                                 // the partial last tile
+                if (n_full & 1) land_and_issue(n_full, pg_b);
+                else land_and_issue(n_full, pg_a);
+                if (active) {
+                    while (!try_compute(n_full, lds + (n_full % 3) * kTileBytes, BoolTag<true>())) move_reference();
+                }
+            }
+        } else {
             Tile rg_even, rg_odd;
             const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
             auto issue_tile = [&](int t, int32_t pg_id, Tile& rg) {
@@ -500,7 +617,7 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     SplitParams p = p_in;
     p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
     p.hg_blocks = p.hkv;
-    const size_t lds_bytes = 2 * (size_t)kTileBytes + 16;
+    const size_t lds_bytes = (FP8 ? 2 : 3) * (size_t)kTileBytes + 16;    // staged tiles: see kDirect
     const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
     // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
