@@ -63,7 +63,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).  e4m3 caches pass
     // through registers for the conversion (two staged tiles).
     constexpr bool kDirect = !FP8;
-    constexpr int kStaged = kDirect ? 3 : 2;   // staged tiles in LDS
+    constexpr int kStaged = kDirect ? 4 : 2;   // staged tiles in LDS
     static_assert(!kDirect || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
                   "direct loads: a first segment of 1 KB per row, a second K segment of 128 bytes");
     constexpr int kK0Row = kDirect ? RK::D0 * 2 : RBK;                 // bytes from one staged row's first K segment to the next row's
@@ -112,15 +112,22 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // lane at 576 values, kept for the whole piece (read from LDS per tile instead, they doubled the LDS traffic of
         // the QK product, which is what bounds it).  Columns past the group repeat its last head; their results are
         // never stored.
-        uint4 qreg[KS];
+        // (Direct loads: the two wavefronts of a tile of 16 q heads share the dot products as well - the one with the even
+        // k-steps, the other with the odd ones, KQ = KS / 2 each - and exchange their halves through LDS: half the reads of
+        // the staged K rows, half the Q^T registers.)
+        constexpr int KQ = kDirect ? KS / CS : KS;                  // k-steps of this wavefront: ks = kq_step * i + kq_first
+        constexpr int kq_step = kDirect ? CS : 1;
+        const int kq_first = kDirect ? whalf : 0;
+        static_assert(!kDirect || (KS % CS == 0 && CS == 2), "the k-steps split by parity");
+        uint4 qreg[KQ];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qreg[ks] = make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < KQ; ++i) qreg[i] = make_uint4(0, 0, 0, 0);
         auto load_q = [&]() {
             if (active) {
                 const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)b * p.q_sb +
-                                     (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a;
+                                     (int64_t)(head0 + min(c, heads_here - 1)) * p.q_sh + 8 * a + 32 * kq_first;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qp + 32 * ks);
+                for (int i = 0; i < KQ; ++i) qreg[i] = *reinterpret_cast<const uint4*>(qp + 32 * kq_step * i);
             }
         };
         if (!kDirect) load_q();                 // (direct loads: requested behind the first rows, see the tile loop)
@@ -373,11 +380,9 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             m_ref = m_new;
         };
 
-        // One tile.  False: a logit of the tile exceeds the reference by more than the slack; nothing has been changed.
-        auto try_compute = [&](int t, const char* buf, auto masked_tag) {
-            constexpr bool MASKED = decltype(masked_tag)::value;
-            const int tok0 = c_start + t * kTile;
-            // Where this lane reads its MFMA operands in the staged tile.  The swizzle XORs the low bits of the
+        // The two halves of a tile's arithmetic: qk_tile, the dot products q . k of the tile's tokens with this wavefront's
+        // heads, and softmax_pv, everything after them.
+        // Where a lane reads its MFMA operands in the staged tile.  The swizzle XORs the low bits of the
             // 16-byte chunk index with the low bits of the row, so the chunks of one lane are 128 bytes apart within
             // each class of the low bits: two base addresses for K (k-steps of either parity), four for V (output blocks
             // modulo four), and constant steps - not one address per operand, which at 18 k-steps and 32 output blocks
@@ -385,17 +390,16 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             //   K operand of k-step ks: row c, chunk 4 ks + a  ->  chunk ^ (c & 7) = 8 (ks >> 1) + ((4 (ks & 1) + a) ^ (c & 7))
             //   V operand of block db (transposed read): row 4 a + (c >> 2), chunk 2 db + ((c & 3) >> 1)
             //                                            ->  2 (4 (db >> 2) + ((db & 3) ^ (row & 3))) + ((c & 3) >> 1)
+        auto qk_tile = [&](const char* buf) {
+            if constexpr (kDirect) {
+                return f32x4_t{0.f, 0.f, 0.f, 0.f};     // (not used: qk_half)
+            } else {
             const char* lk = buf + c * kK0Row;
             const char* k_at[2] = {lk + (((0 + a) ^ (c & 7)) << 4), lk + (((4 + a) ^ (c & 7)) << 4)};
             // (k-steps of the second K segment: from row c's second segment on, which in the direct-load layout lies
             // elsewhere than behind its first)
             constexpr int KSEG0 = RK::D0 / 32;
             const int k1_delta = kK1Base + c * (kK1Row - kK0Row) - KSEG0 / 2 * 128;
-            const int k4 = c >> 2, cc = c & 3;
-            const int vrow = 4 * a + k4;
-            const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8 + whalf * (DB / 4) * 128;   // (+ this wavefront's columns)
-            const char* v_at[4] = {lv + ((0 ^ (vrow & 3)) << 5), lv + ((1 ^ (vrow & 3)) << 5), lv + ((2 ^ (vrow & 3)) << 5),
-                                   lv + ((3 ^ (vrow & 3)) << 5)};
             // ---- S^T[token][head] = K Q^T: QG accumulation chains; the K operands of the next QG k-steps are requested
             // from LDS before the MFMA of the current ones (and no further ahead: every operand held in registers is
             // one the output tile and the loads under way cannot have) ----
@@ -424,6 +428,43 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             f32x4_t s = s3[0];
 #pragma unroll
             for (int i = 1; i < QG; ++i) s += s3[i];
+            return s;
+            }
+        };
+        // Direct loads: this wavefront's half of the dot products, k-steps kq_first, kq_first + 2, ...: the operands of its
+        // parity class are 128 bytes apart from ONE base address (the last k-step lies in the second K segment).
+        auto qk_half = [&](const char* buf) {
+            constexpr int KSEG0 = RK::D0 / 32;
+            const char* k_at = buf + c * kK0Row + (((4 * kq_first + a) ^ (c & 7)) << 4);
+            const int k1_delta = kK1Base + c * (kK1Row - kK0Row) - KSEG0 / 2 * 128;
+            constexpr int QG = 3, NQG = KQ / QG;
+            static_assert(KQ % QG == 0, "k-steps in whole groups");
+            f32x4_t s3[QG];
+#pragma unroll
+            for (int i = 0; i < QG; ++i) s3[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            uint4 ka[KQ];
+#pragma unroll
+            for (int i = 0; i < KQ; ++i)        // (k-step 2 i + kq_first: chunk group i; from KSEG0 on in the second segment)
+                ka[i] = *reinterpret_cast<const uint4*>(k_at + (2 * i >= KSEG0 ? k1_delta : 0) + i * 128);
+#pragma unroll
+            for (int g = 0; g < NQG; ++g) {
+#pragma unroll
+                for (int i = 0; i < QG; ++i) s3[i] = M::qk(ka[g * QG + i], qreg[g * QG + i], s3[i]);
+            }
+            f32x4_t s = s3[0];
+#pragma unroll
+            for (int i = 1; i < QG; ++i) s += s3[i];
+            return s;
+        };
+        // False: a logit of the tile exceeds the reference by more than the slack; nothing has been changed.
+        auto softmax_pv = [&](int t, const char* buf, const f32x4_t s, auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            const int tok0 = c_start + t * kTile;
+            const int k4 = c >> 2, cc = c & 3;
+            const int vrow = 4 * a + k4;
+            const char* lv = buf + kTile * RBK + vrow * RBV + (cc >> 1) * 16 + (cc & 1) * 8 + whalf * (DB / 4) * 128;   // (+ this wavefront's columns)
+            const char* v_at[4] = {lv + ((0 ^ (vrow & 3)) << 5), lv + ((1 ^ (vrow & 3)) << 5), lv + ((2 ^ (vrow & 3)) << 5),
+                                   lv + ((3 ^ (vrow & 3)) << 5)};
             float sv[4] = {s.x, s.y, s.z, s.w};
             if (softcap) {
 #pragma unroll
@@ -469,6 +510,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             }
             return true;
         };
+        auto try_compute = [&](int t, const char* buf, auto masked_tag) { return softmax_pv(t, buf, qk_tile(buf), masked_tag); };
 
         // ---- the tiles of the piece: the loads of tiles t + 1 and t + 2 are under way while all wavefronts work on tile t
         // (two register tiles by the parity of t; the memory system's latency is longer than the arithmetic of one tile).
@@ -477,58 +519,89 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // (A wavefront that leaves the inner loop to move its reference does so after the tile's barrier and comes back for
         // the next tile: every wavefront passes exactly one barrier per tile.) ----
         if constexpr (kDirect) {
-            // Direct loads, three staged tiles: tile t is read from buffer t % 3 while the loads of tiles t + 1 and t + 2 are
-            // under way into the other two.  Per tile: wait until this wavefront's loads of tile t have landed, barrier
-            // (every wavefront's have, and every wavefront has finished with tile t - 1), request tile t + 2 into the buffer
-            // of tile t - 1, work on tile t.  Every wavefront issues exactly kLoadsPerTile loads per tile, and loads return
-            // in order: "tile t has landed" is "at most kLoadsPerTile loads under way" while tile t + 1 has been requested,
-            // "none under way" for the last tile.  (Loads that the compiler sees - page numbers per row, PM_ROW - only make
-            // these waits, and the compiler's own, wait for more than they need.)
+            // Direct loads, four staged tiles (tile t in buffer t % 4), and the arithmetic of two tiles in one step: the dot
+            // products of tile t + 1 next to the softmax and the PV product of tile t, which do not depend on each other - the
+            // matrix cores work on the one while the vector ALU and the LDS round trips of the other are under way (with one
+            // tile per step a wavefront's MFMA, softmax and MFMA again each wait for the one before).
+            // Step t: wait until this wavefront's loads of tile t + 1 have landed; barrier (every wavefront's have, and every
+            // wavefront is done with tile t - 1); request tile t + 3 into the buffer of tile t - 1; q . k of tile t + 1,
+            // softmax and PV of tile t.  Loads return in order and every wavefront issues kLoadsPerTile of them per tile:
+            // "tile t + 1 has landed" is "at most kLoadsPerTile loads under way" while tile t + 2 has been requested, "none
+            // under way" otherwise.  (Loads that the compiler sees - page numbers per row, PM_ROW - only make these waits,
+            // and the compiler's own, wait for more than they need.)
             const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
+            auto staged = [&](int t) { return lds + (t & 3) * kTileBytes; };
             auto issue_tile = [&](int t, int32_t pg_id) {
-                const uint32_t dst = lds0 + (uint32_t)(t % 3) * kTileBytes;
+                const uint32_t dst = lds0 + (uint32_t)(t & 3) * kTileBytes;
                 if (t < n_full) issue_direct(BoolTag<false>(), t, pg_id, dst);
                 else if (t < n_tiles) issue_direct(BoolTag<true>(), t, pg_id, dst);
             };
             // the staged tiles are free: no wavefront still reads the previous piece's, none of its loads is under way
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            int32_t pg_a = page_id(2), pg_b = page_id(3);           // (a: even tiles, b: odd tiles)
             issue_tile(0, page_id(0));
             issue_tile(1, page_id(1));
+            issue_tile(2, page_id(2));
+            int32_t pg_hold = page_id(3);
             load_q();
             // Q^T has to have arrived HERE: the compiler would otherwise wait for its loads where they are first used, inside
             // the tile loop, by counting down to "no load under way" - in every iteration, and the rows requested for the
             // tiles ahead are loads it does not know of.  (An empty asm that takes the registers as operands is such a use.)
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qreg[ks].x), "+v"(qreg[ks].y), "+v"(qreg[ks].z), "+v"(qreg[ks].w));
-            auto land_and_issue = [&](int t, int32_t& pg) {
-                static_assert(kLoadsPerTile == 5, "the wait below counts the loads of one tile");
-                if (t + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(5)\n\ts_barrier" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-                const int32_t pg_now = pg;
-                pg = page_id(t + 4);
-                issue_tile(t + 2, pg_now);
+            for (int i = 0; i < KQ; ++i) asm volatile("" : "+v"(qreg[i].x), "+v"(qreg[i].y), "+v"(qreg[i].z), "+v"(qreg[i].w));
+            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");          // tile 0 is there
+            static_assert(kLoadsPerTile == 5, "the wait below counts the loads of one tile");
+            // (the barrier also waits for this wavefront's LDS operations: its half of the next tile's dot products is in
+            // the exchange area, its reads of the partner's half of the tile before are done)
+            auto step = [&](int t) {
+                if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                const int32_t pg_now = pg_hold;
+                pg_hold = page_id(t + 4);
+                issue_tile(t + 3, pg_now);
             };
+            // The halves of a tile's dot products cross between the two wavefronts of a head tile through the exchange area
+            // behind the staged tiles: [tile parity][wavefront][lane] x 16 bytes.  A wavefront writes its half of tile t + 1
+            // in step t and reads the partner's after the barrier of step t + 1; the same place is written again in step
+            // t + 2, after a barrier that the partner reaches only when that read is done.
+            char* const xch = lds + kStaged * kTileBytes + 16;
+            auto put_half = [&](int t, const f32x4_t s) {
+                *reinterpret_cast<float4*>(xch + (((t & 1) * NW + wave) * 64 + lane) * 16) = make_float4(s.x, s.y, s.z, s.w);
+            };
+            auto whole = [&](int t, const f32x4_t mine) {
+                const float4 o = *reinterpret_cast<const float4*>(xch + (((t & 1) * NW + (wave ^ 1)) * 64 + lane) * 16);
+                return f32x4_t{mine.x + o.x, mine.y + o.y, mine.z + o.z, mine.w + o.w};
+            };
+            f32x4_t s_mine = {0.f, 0.f, 0.f, 0.f}, s_cur = {0.f, 0.f, 0.f, 0.f};
+            if (active) {
+                s_mine = qk_half(staged(0));
+                put_half(0, s_mine);
+            }
             int t = 0;
             for (;;) {
                 bool gave_up = false;
                 for (; t < n_full; ++t) {
-                    if (t & 1) land_and_issue(t, pg_b);
-                    else land_and_issue(t, pg_a);
-                    if (active && !try_compute(t, lds + (t % 3) * kTileBytes, BoolTag<false>())) {
-                        gave_up = true;
-                        break;
+                    step(t);
+                    if (active) {
+                        s_cur = whole(t, s_mine);
+                        if (t + 1 < n_tiles) {
+                            s_mine = qk_half(staged(t + 1));
+                            put_half(t + 1, s_mine);
+                        }
+                        if (!softmax_pv(t, staged(t), s_cur, BoolTag<false>())) {
+                            gave_up = true;
+                            break;
+                        }
                     }
                 }
                 if (!gave_up) break;
-                do move_reference(); while (!try_compute(t, lds + (t % 3) * kTileBytes, BoolTag<false>()));
+                do move_reference(); while (!softmax_pv(t, staged(t), s_cur, BoolTag<false>()));
                 ++t;
             }
             if (n_full < n_tiles) {                                 // the partial last tile
-                if (n_full & 1) land_and_issue(n_full, pg_b);
-                else land_and_issue(n_full, pg_a);
+                step(n_full);
                 if (active) {
-                    while (!try_compute(n_full, lds + (n_full % 3) * kTileBytes, BoolTag<true>())) move_reference();
+                    s_cur = whole(n_full, s_mine);
+                    while (!softmax_pv(n_full, staged(n_full), s_cur, BoolTag<true>())) move_reference();
                 }
             }
         } else {
@@ -617,7 +690,8 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     SplitParams p = p_in;
     p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
     p.hg_blocks = p.hkv;
-    const size_t lds_bytes = (FP8 ? 2 : 3) * (size_t)kTileBytes + 16;    // staged tiles: see kDirect
+    // staged tiles, the next work item, and (direct loads) the exchange area of the half dot products: see kDirect
+    const size_t lds_bytes = FP8 ? 2 * (size_t)kTileBytes + 16 : 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024;
     const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
     // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
