@@ -7,20 +7,30 @@
 // the memory system is the limit (G <= 16: every row is read once).  At G = 128 it is not: the rows cross the L2 eight
 // times and the matrix cores idle.  Here the wavefronts of a workgroup take DIFFERENT q-head tiles of the SAME kv head
 // and the same tokens: a tile of K / V rows is loaded once by the workgroup (each wavefront loads its share of the
-// rows), staged once in LDS, and every wavefront multiplies it with its own 16 q heads.  Two staged tiles alternate,
-// so one barrier per tile is enough: a wavefront writes tile t + 1 only after the barrier of tile t, which every
-// wavefront reaches after it has finished reading tile t - 1 from the same buffer.
+// rows), staged once in LDS, and every wavefront multiplies it with its own 16 q heads.
 //
 // A workgroup covers kSharedTileHeads = 64 q heads with eight wavefronts: two per tile of 16 q heads, each of which
-// forms the tile's logits and softmax for itself and accumulates one half of the output columns (64 accumulation
-// registers per lane at 512 values; Q^T takes 72 more), two wavefronts per SIMD.  A group of 128 q heads is two such
-// workgroups, which the launch places on one XCD (tiles_on_one_xcd).  Same arithmetic per (q head, token) as the other
-// kernels (fdk_splitkv_mfma_body.h): S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with
-// 16x16x16 MFMA and P rounded to the cache dtype; the QK product runs as six interleaved accumulation chains (18
-// dependent MFMA would wait for each other), and the running maximum of the softmax is a reference that moves rarely,
-// so that the tile loop holds no rescale of the output tile (see move_reference).  16-bit and e4m3 caches; page numbers per tile
-// or per row (PM_TILE, PM_ROW).  How pieces are handed out is shared with the other kernels
-// (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
+// forms the tile's softmax for itself and accumulates one half of the output columns (64 accumulation registers per
+// lane at 512 values), two wavefronts per SIMD.  A group of 128 q heads is two such workgroups, which the launch places
+// on one XCD (tiles_on_one_xcd).  Same arithmetic per (q head, token) as the other kernels (fdk_splitkv_mfma_body.h):
+// S^T = K Q^T with 16x16x32 MFMA, online softmax in fp32, O^T += V^T P^T with 16x16x16 MFMA and P rounded to the cache
+// dtype; the running maximum of the softmax is a reference that moves rarely, so that the tile loop holds no rescale of
+// the output tile (see move_reference).  Page numbers per tile or per row (PM_TILE, PM_ROW).  How pieces are handed out
+// is shared with the other kernels (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
+//
+// 16-bit caches (kDirect): the rows never pass through registers.  global_load_lds_dwordx4 writes the 16 bytes of lane i
+// to LDS byte M0 + 16 i, so a load instruction fills 1 KB of a staged tile directly; the swizzle of the staged rows is
+// applied on the memory side (the lane whose bytes land in chunk x of row r fetches chunk x ^ swizzle(r) of that row).
+// Four staged tiles: tile t is worked on while tiles t + 1 ... t + 3 land.  The compiler would put "wait for every load
+// under way" in front of each LDS read that follows such a load, so the loads are issued from inline asm and the tile
+// loop waits by count itself (loads return in order, every wavefront issues five per tile).  The two wavefronts of a
+// head tile also split the q . k products - even and odd k-steps, nine each, 36 registers of Q^T each - and exchange
+// their halves through LDS; a step of the loop holds the half dot products of tile t + 1 next to the softmax and the PV
+// product of tile t, which do not depend on each other, and ONE barrier.
+// e4m3 caches: the rows pass through registers for the conversion (each wavefront loads its share two tiles ahead and
+// stores it, converted, into one of two staged tiles; one barrier per tile: a wavefront writes tile t + 1 only after
+// the barrier of tile t, which every wavefront reaches after it has finished reading tile t - 1 from the same buffer);
+// every wavefront forms all of its head tile's dot products (six interleaved accumulation chains, Q^T in 72 registers).
 #pragma once
 
 #include "fdk_splitkv_mfma.h"
@@ -48,7 +58,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr bool kOneSegment = false;        // (fdk_splitkv_mfma_work.h: several head tiles of a kv head go to one XCD)
     constexpr bool kRowsShareLines = false;    // (16-bit rows: whole 128-byte lines per kv head)
     constexpr int kTileHeads = kSharedTileHeads;
-    constexpr bool kFirstPieceStraight = false; // (fdk_splitkv_mfma_work.h: one copy of the piece, which needs every register)
+    constexpr bool kFirstPieceStraight = !FP8;  // (fdk_splitkv_mfma_work.h; e4m3: one copy of the piece, which needs every register)
     constexpr int NW = kSharedWaves;
     constexpr int ES = FP8 ? 1 : 2;            // bytes per cache value
     constexpr int RBK = 2 * DK, RBV = 2 * DV;  // bytes of a staged row
@@ -57,7 +67,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr int DB = DV / 16 / CS;           // 16-column blocks of the output that this wavefront holds
     constexpr int kTileBytes = kTile * (RBK + RBV);
     // 16-bit caches: the rows go from memory straight into the staged tile (global_load_lds_dwordx4: lane i of a load
-    // instruction writes its 16 bytes at M0 + 16 i, no registers in between and nothing to store), three staged tiles.
+    // instruction writes its 16 bytes at M0 + 16 i, no registers in between and nothing to store), four staged tiles.
     // A load instruction then fills 1 KB of consecutive LDS, so the second K segment of the 16 rows lies behind their
     // first segments instead of behind each row, and the swizzle is applied on the memory side: the lane whose bytes
     // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).  e4m3 caches pass
@@ -73,7 +83,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr int KS0 = (RK::NJ0 + NW - 1) / NW, KS1 = (RK::NJ1 + NW - 1) / NW;
     constexpr int VS0 = (RV::NJ0 + NW - 1) / NW, VS1 = (RV::NJ1 + NW - 1) / NW;
 
-    extern __shared__ __attribute__((aligned(16))) char lds[];      // two staged tiles, then the next work item
+    extern __shared__ __attribute__((aligned(16))) char lds[];      // the staged tiles, the next work item, (kDirect) the exchange area
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
