@@ -644,11 +644,15 @@ def test_head_dims_of_two_segments_and_v_rows_of_their_own_length():
 
 def test_plans_of_wide_rows_keep_to_what_a_compute_unit_holds():
     # blocks of 4 or 8 kv heads are eight wavefronts; rows of more than 512 values per token and kv head (K and V
-    # together) leave registers and LDS for four, i.e. at most two heads per workgroup
+    # together): 16-bit caches run in the kernels whose wavefronts share the staged tiles, one kv head per workgroup
+    # whatever the group; e4m3 caches with at most 16 q heads per kv head in the 16-head kernels, whose registers and
+    # LDS hold four wavefronts, i.e. at most two heads per workgroup
     big = dict(batch=512, max_kv_len=2048, min_kv_len=2048)
     assert _plan(_dims(192, 192, **big)).kv_heads_per_wg == 8
     assert _plan(_dims(192, 128, **big)).kv_heads_per_wg == 8
     p = _plan(_dims(576, 512, **big))
+    assert p.kv_heads_per_wg == 1 and p.num_splits == 1
+    p = _plan(_dims(576, 512, kv_dtype=_lib.FDK_FP8_E4M3, **big))
     assert p.kv_heads_per_wg == 2 and p.num_splits == 1
     # large q-head groups on one kv head of 576 + 512 values: one kv head and 64 q heads per workgroup (the kernels whose
     # wavefronts share the staged tiles), so 32 sequences x 128 q heads are 64 units and split four ways on 256 compute units

@@ -302,12 +302,12 @@ def test_two_segment_head_dims_in_every_plan(cuda_device, dims, page):
     check(out_q, lse_q, "work queue")
     check(out_f, lse_f, "fp32 out")
     torch.testing.assert_close(out_f, out_b.float(), atol=1e-2, rtol=1e-2)
-    # a batch that fills the GPU by itself: whole sequences per workgroup, in blocks of kv heads (at most two heads per
-    # workgroup where a token's K and V rows hold more than 512 values)
+    # a batch that fills the GPU by itself: whole sequences per workgroup, in blocks of kv heads (one head per workgroup
+    # where a token's K and V rows hold more than 512 values: the kernels whose wavefronts share the staged tiles)
     lens2 = [int(x) for x in torch.randint(40, 160, (130,), generator=g)]
     q2, k2, v2, table2, lens2_t = _two_segment_inputs(cuda_device, dims, lens2, (16, 8), page, torch.float16, 99 + page)
     plan2 = tda.get_split_kv_plan(q2, k2, v2, table2, lens2_t, scale, max_kv_len=max(lens2), min_kv_len=max(lens2))
-    assert plan2.num_splits == 1 and plan2.kv_heads_per_wg == (2 if dk + dv > 512 else 4), plan2
+    assert plan2.num_splits == 1 and plan2.kv_heads_per_wg == (1 if dk + dv > 512 else 4), plan2
     o2, l2 = tda.flash_decode(q2, k2, v2, table2, lens2_t, scale, max_kv_len=max(lens2), min_kv_len=max(lens2))
     torch.cuda.synchronize()
     _check(o2, l2, q2, k2, v2, table2, lens2, scale, tag=f"dims={dims} P={page} single pass")
@@ -489,7 +489,7 @@ def test_two_segment_head_dims_random_shapes_with_an_fp8_cache(cuda_device, seed
 def test_two_segment_head_dims_with_an_fp8_cache(cuda_device, dims, heads, page):
     """e4m3 caches with per-kv-head scales behind rows of two segments: exact dequantisation (the decode over the
     dequantised cache) and the K scale folded into the logit scale, through a single pass, chunks, a work queue and equal
-    shares; groups of more than 32 q heads on rows of 576 / 512 values run in the kernels that share the staged tiles.
+    shares; groups of more than 16 q heads on rows of 576 / 512 values run in the kernels that share the staged tiles.
     fp16 queries at page size 6."""
     dk, dv = dims
     hq, hkv = heads

@@ -282,9 +282,9 @@ int make_plan(const fdk_decode_args* a, int num_cus, fdk_plan_t* plan) {
     const bool heads_contiguous = a->k_stride_head == a->head_dim && a->v_stride_head == a->head_dim;
     int kv_heads_per_wg = 1;
     int units_per_seq;
-    const int tile_heads = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a)) : 16;   // q heads of a kv head per workgroup
+    const int tile_heads = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a), a->kv_dtype) : 16;   // q heads of a kv head per workgroup
     if (algo == FDK_ALGO_MFMA) {
-        kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus, a->head_dim + v_dim(a));
+        kv_heads_per_wg = fdk::mfma_kv_heads_per_wg(batch, a->num_kv_heads, group, num_cus, a->head_dim + v_dim(a), a->kv_dtype);
         units_per_seq = fdk::mfma_units_per_seq(a->num_kv_heads, group, kv_heads_per_wg, tile_heads);
     } else {
         units_per_seq = fdk::valu_units_per_seq(a->num_kv_heads, group, heads_contiguous, a->kv_dtype);
@@ -441,7 +441,7 @@ int piece_cost_granules(const fdk_decode_args* a, int kv_heads_per_wg) {
 // q-head tiles per kv head, as the resolved algorithm's kernel counts them
 int head_tiles_of(const fdk_decode_args* a, int algo) {
     const int group = a->num_q_heads / a->num_kv_heads;
-    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a)) : fdk::valu_heads_per_wg(group);
+    const int hpw = algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(group, a->head_dim + v_dim(a), a->kv_dtype) : fdk::valu_heads_per_wg(group);
     return (group + hpw - 1) / hpw;
 }
 
@@ -498,7 +498,7 @@ int resolve(const fdk_decode_args* a, bool direct_ok, int num_cus, Resolved* r) 
     sp.hg_per_wg = r->plan.kv_heads_per_wg;
     sp.balanced = r->plan.balanced;
     sp.workgroups = r->plan.workgroups;
-    sp.tile_heads = r->plan.algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(sp.group, a->head_dim + v_dim(a)) : 16;
+    sp.tile_heads = r->plan.algo == FDK_ALGO_MFMA ? fdk::mfma_heads_per_wg(sp.group, a->head_dim + v_dim(a), a->kv_dtype) : 16;
     sp.heads_per_tile = sp.group < sp.tile_heads ? sp.group : sp.tile_heads;
     sp.rows_per_slot = sp.hg_per_wg * sp.heads_per_tile;
     sp.piece_cost = sp.balanced ? piece_cost_granules(a, sp.hg_per_wg) : 0;

@@ -148,8 +148,8 @@ bool valu_supported(int q_dtype, int kv_dtype, int group, int head_dim);
 int valu_units_per_seq(int hkv, int group, bool heads_contiguous, int kv_dtype);
 bool mfma_supported(int q_dtype, int kv_dtype, int group, int head_dim, int v_head_dim);
 int valu_heads_per_wg(int group);
-int mfma_heads_per_wg(int group, int row_values);   // q heads of a kv head per workgroup (SplitParams.tile_heads)
-int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values);   // row_values: head_dim + v_head_dim
+int mfma_heads_per_wg(int group, int row_values, int kv_dtype);   // q heads of a kv head per workgroup (SplitParams.tile_heads)
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values, int kv_dtype);   // row_values: head_dim + v_head_dim
 int mfma_units_per_seq(int hkv, int group, int kv_heads_per_wg, int tile_heads);
 
 #if defined(__HIPCC__)

@@ -453,7 +453,9 @@ int launch_mfma_rows2(const SplitParams& p, int q_dtype, int kv_dtype, hipStream
     if (kv_dtype == FDK_FP8_E4M3)
         return q_dtype == FDK_BF16 ? launch_rows2<FDK_BF16, DK, DV, MODE, true>(p, stream) : launch_rows2<FDK_FP16, DK, DV, MODE, true>(p, stream);
     if (kv_dtype != q_dtype) return (int)hipErrorInvalidValue;
-    return q_dtype == FDK_BF16 ? launch_rows2<FDK_BF16, DK, DV, MODE, false>(p, stream) : launch_rows2<FDK_FP16, DK, DV, MODE, false>(p, stream);
+    // (16-bit caches with rows of more than 512 values run in the shared-tile kernels whatever the group: mfma_heads_per_wg)
+    if constexpr (DK + DV > 512) return (int)hipErrorInvalidValue;
+    else return q_dtype == FDK_BF16 ? launch_rows2<FDK_BF16, DK, DV, MODE, false>(p, stream) : launch_rows2<FDK_FP16, DK, DV, MODE, false>(p, stream);
 }
 
 template <int D, int MODE>

@@ -37,11 +37,15 @@ bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim, int 
     return two_segments && (kv_dtype == q_dtype || kv_dtype == FDK_FP8_E4M3);
 }
 
-// q heads of one kv head that a workgroup covers: a tile of 16 (a wavefront per kv head), or 64 where the rows are
-// long and the group is large - latent attention, 128 q heads on one kv head of 576 + 512 values - and the kernels of
-// fdk_splitkv_mfma_shared.h load and stage every tile once for four tiles of 16 q heads
-int mfma_heads_per_wg(int group, int row_values) {
-    return row_values > 512 && group > 32 ? 64 : 16;
+// q heads of one kv head that a workgroup covers: a tile of 16 (a wavefront per kv head), or 64 where the rows are long -
+// latent attention, up to 128 q heads on one kv head of 576 + 512 values - and the kernels of fdk_splitkv_mfma_shared.h
+// load and stage every tile once for four tiles of 16 q heads.  16-bit caches: whatever the group, the rows of those
+// kernels go straight from memory into LDS, which beats the 16-head kernels even where most of a workgroup's wavefronts
+// have no q heads and only help to load (batch 32 x 4096 tokens, 8 / 16 / 32 q heads: 51 / 52 / 56 us against 75 / 77 /
+// 115 us).  e4m3 caches pass through registers either way: from 17 q heads on (8 / 16 / 32 q heads: 58 / 59 / 66 us
+// against 50 / 52 / 90 us).
+int mfma_heads_per_wg(int group, int row_values, int kv_dtype) {
+    return row_values > 512 && (kv_dtype != FDK_FP8_E4M3 || group > 16) ? 64 : 16;
 }
 
 // kv heads per workgroup.  Adjacent kv heads of a token are adjacent in the cache, so a workgroup that takes
@@ -55,8 +59,8 @@ int mfma_heads_per_wg(int group, int row_values) {
 // the number of independent workgroups.
 // (Rows of more than 512 values per token and kv head, K and V together: at most two heads, i.e. the four wavefronts
 // that the registers and the LDS of a compute unit hold at that size.)
-int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values) {
-    if (mfma_heads_per_wg(group, row_values) > 16) return 1;   // the shared-tile kernels: one kv head, 64 q heads
+int mfma_kv_heads_per_wg(int batch, int hkv, int group, int num_cus, int row_values, int kv_dtype) {
+    if (mfma_heads_per_wg(group, row_values, kv_dtype) > 16) return 1;   // the shared-tile kernels: one kv head, 64 q heads
     const int head_tiles = (group + 15) / 16;
     for (int nh = row_values > 512 ? 2 : 8; nh >= 1; nh >>= 1) {
         if (hkv % nh) continue;
