@@ -257,6 +257,64 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j, 0, byte, byte, vplane, vsp_bytes, vst_bytes), dst + kTile * RBK + j * 1024);
             }
         };
+        // Page numbers per row (PM_ROW) for the direct loads.  A vector load that the compiler sees would make it wait, in
+        // front of the first use of the numbers, for every row requested since - so they take the same road as the rows:
+        // global_load_lds_dword puts the page numbers of a tile's 16 rows (lane i: row i & 15; rows past the end repeat the
+        // last token) into one of eight slots behind the exchange area, and the requests for the rows read them from there,
+        // by then long landed (see the tile loop).  All wavefronts write the same numbers to the same place.
+        constexpr int kPageSlots = 8;
+        const uint32_t pg_lds = (uint32_t)(kStaged * kTileBytes + 16 + 2 * NW * 1024);    // offset of the slots from lds[0]
+        auto issue_pages = [&](int t) {
+            const int n = min(c_start + t * kTile + (lane & 15), c_end - 1);
+            const int idx = p.page_shift < 0 ? n / p.page_size : n >> p.page_shift;
+            const int32_t* ptr = p.block_table + (int64_t)b * p.tbl_sb + idx;
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(ptr), "s"(lds0 + pg_lds + (uint32_t)(t & (kPageSlots - 1)) * 256)
+                         : "memory");
+        };
+        // Tile t with page numbers per row.  A first-segment instruction covers ONE row: its page number, read from the slot
+        // by every lane alike, its place in the page and with them its address are wave-uniform.  The instruction of the
+        // second K segment covers eight rows: a lane reads the number of its own.
+        auto issue_direct_rows = [&](int t, uint32_t dst) {
+            const int tok0 = c_start + t * kTile;
+            const int32_t* pages = reinterpret_cast<const int32_t*>(lds + pg_lds + (t & (kPageSlots - 1)) * 256);
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            ln &= 63;
+            auto place = [&](int n) { return p.page_shift < 0 ? (uint32_t)(n % p.page_size) : (uint32_t)(n & pmask); };
+            // (all page numbers first: every request for rows is an asm statement that no LDS read may cross, and a read
+            // in front of each would cost its round trip each time)
+            static_assert(KS0 == VS0 && RK::NJ0 == RV::NJ0 && KS1 <= 1, "K and V rows of the first segments pair up");
+            int32_t pg_row[KS0], pg_lane = 0;
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) pg_row[s] = pages[slot_instr(s, RK::NJ0)];
+            const int j1 = slot_instr(0, RK::NJ1 > 0 ? RK::NJ1 : 1);
+            if (KS1) pg_lane = pages[j1 * 8 + (ln >> 3)];
+            uint64_t k_base[KS0], v_base[KS0];                      // wave-uniform: page and place of the row
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int n = min(tok0 + slot_instr(s, RK::NJ0), c_end - 1);
+                const uint32_t pg = (uint32_t)__builtin_amdgcn_readfirstlane(pg_row[s]);
+                const uint32_t pl = place(n);
+                k_base[s] = (uint64_t)pg * ksp_bytes + (uint64_t)(pl * kst_bytes);
+                v_base[s] = (uint64_t)pg * vsp_bytes + (uint64_t)(pl * vst_bytes);
+            }
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                load_to_lds16(kplane + k_base[s] + (uint32_t)((ln ^ (j & 7)) << 4), dst + j * 1024);
+            }
+            if (KS1) {
+                const int n = min(tok0 + j1 * 8 + (ln >> 3), c_end - 1);
+                const uint32_t byte = (uint32_t)(RK::D0 * ES + (((ln & 7) ^ ((ln >> 3) & 7)) << 4));
+                load_to_lds16(kplane + ((uint64_t)(uint32_t)pg_lane * ksp_bytes + (uint64_t)(place(n) * kst_bytes)) + byte,
+                              dst + kK1Base + j1 * 1024);
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                load_to_lds16(vplane + v_base[s] + (uint32_t)((ln ^ ((j & 3) << 1)) << 4), dst + kTile * RBK + j * 1024);
+            }
+        };
         auto issue = [&](auto clamp_tag, int t, int32_t pg_id, Tile& rg) {
             const int tok0 = c_start + t * kTile;
             int ln = lane;                                  // (as in stage below)
@@ -543,15 +601,31 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             auto staged = [&](int t) { return lds + (t & 3) * kTileBytes; };
             auto issue_tile = [&](int t, int32_t pg_id) {
                 const uint32_t dst = lds0 + (uint32_t)(t & 3) * kTileBytes;
-                if (t < n_full) issue_direct(BoolTag<false>(), t, pg_id, dst);
-                else if (t < n_tiles) issue_direct(BoolTag<true>(), t, pg_id, dst);
+                if (PM == PM_ROW) {
+                    if (t < n_tiles) issue_direct_rows(t, dst);
+                } else if (t < n_full) {
+                    issue_direct(BoolTag<false>(), t, pg_id, dst);
+                } else if (t < n_tiles) {
+                    issue_direct(BoolTag<true>(), t, pg_id, dst);
+                }
             };
             // the staged tiles are free: no wavefront still reads the previous piece's, none of its loads is under way
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            issue_tile(0, page_id(0));
-            issue_tile(1, page_id(1));
-            issue_tile(2, page_id(2));
-            int32_t pg_hold = page_id(3);
+            int32_t pg_hold = 0;
+            if (PM == PM_ROW) {
+                // page numbers per row come through LDS as well (issue_pages), two steps ahead of the rows that need them
+#pragma unroll
+                for (int t = 0; t < 5; ++t) issue_pages(t);
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                issue_tile(0, 0);
+                issue_tile(1, 0);
+                issue_tile(2, 0);
+            } else {
+                issue_tile(0, page_id(0));
+                issue_tile(1, page_id(1));
+                issue_tile(2, page_id(2));
+                pg_hold = page_id(3);
+            }
             load_q();
             // Q^T has to have arrived HERE: the compiler would otherwise wait for its loads where they are first used, inside
             // the tile loop, by counting down to "no load under way" - in every iteration, and the rows requested for the
@@ -559,15 +633,25 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
 #pragma unroll
             for (int i = 0; i < KQ; ++i) asm volatile("" : "+v"(qreg[i].x), "+v"(qreg[i].y), "+v"(qreg[i].z), "+v"(qreg[i].w));
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");          // tile 0 is there
-            static_assert(kLoadsPerTile == 5, "the wait below counts the loads of one tile");
+            static_assert(kLoadsPerTile == 5, "the waits below count the loads of one tile");
             // (the barrier also waits for this wavefront's LDS operations: its half of the next tile's dot products is in
             // the exchange area, its reads of the partner's half of the tile before are done)
+            // PM_ROW: a step requests the rows of tile t + 3 and then the page numbers of tile t + 5, one load more; what has
+            // to have landed at the top of step t are the rows of tile t + 1 and the page numbers of tile t + 3, both requested
+            // in step t - 2: everything but the loads of step t - 1, which are six, or the one of the page numbers alone.
             auto step = [&](int t) {
-                if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                const int32_t pg_now = pg_hold;
-                pg_hold = page_id(t + 4);
-                issue_tile(t + 3, pg_now);
+                if (PM == PM_ROW) {
+                    if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    issue_tile(t + 3, 0);
+                    issue_pages(t + 5);
+                } else {
+                    if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(5) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    const int32_t pg_now = pg_hold;
+                    pg_hold = page_id(t + 4);
+                    issue_tile(t + 3, pg_now);
+                }
             };
             // The halves of a tile's dot products cross between the two wavefronts of a head tile through the exchange area
             // behind the staged tiles: [tile parity][wavefront][lane] x 16 bytes.  A wavefront writes its half of tile t + 1
@@ -701,7 +785,7 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
     p.hg_blocks = p.hkv;
     // staged tiles, the next work item, and (direct loads) the exchange area of the half dot products: see kDirect
-    const size_t lds_bytes = FP8 ? 2 * (size_t)kTileBytes + 16 : 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024;
+    const size_t lds_bytes = FP8 ? 2 * (size_t)kTileBytes + 16 : 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 8 * 256;   // (+ page numbers)
     const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
     // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
