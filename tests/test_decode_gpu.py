@@ -439,6 +439,45 @@ def test_large_groups_on_one_kv_head_share_the_staged_tiles(cuda_device, heads, 
     torch.testing.assert_close(packed[live][..., 512].float(), lse_a[live], atol=3e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("heads", [(64, 1), (128, 2), (40, 1), (71, 1), (51, 3)])
+@pytest.mark.parametrize("page", [16, 1, 6])
+def test_large_groups_at_head_dim_128(cuda_device, heads, page):
+    """More than 16 q heads per kv head with rows of 128 values (multi-query attention): the q-head tiles of a kv head run
+    on one XCD and load with plain loads.  Every way of handing out the pieces, empty sequences, fp16, a soft cap, an
+    e4m3 cache, the single-launch form (which stays with the other kernels)."""
+    hq, hkv = heads
+    scale = 128 ** -0.5
+    g = torch.Generator().manual_seed(hq * 5 + hkv + page)
+    lens = [int(x) for x in torch.randint(1, 2500, (6,), generator=g)]
+    lens[1], lens[4] = 0, 1
+    dtype = torch.float16 if page == 1 else torch.bfloat16
+    cap = 30.0 if page == 6 else 0.0
+    q, k, v, table, lens_t = _two_segment_inputs(cuda_device, (128, 128), lens, heads, page, dtype, 700 + hq + page, table_extra=1)
+    live = [i for i, n in enumerate(lens) if n > 0]
+
+    def check(o, l, tag, **kw):
+        assert o.shape == (len(lens), hq, 128)
+        assert torch.isfinite(o.float()).all() and float(o[1].abs().max()) == 0 and bool((l[1] == -math.inf).all()), tag
+        _check(o[live], l[live], q[live], k, v, table[live], [lens[i] for i in live], scale, cap, tag=f"heads={heads} P={page} {tag}", **kw)
+
+    for tag, kw in (("auto", {}), ("single pass", dict(kv_split=1)), ("5 chunks", dict(kv_split=5)), ("queue", dict(kv_split=40)),
+                    ("equal shares", dict(force_balanced=True)), ("alike lengths", dict(max_kv_len=max(lens), min_kv_len=max(lens)))):
+        o, l = tda.flash_decode(q, k, v, table, lens_t, scale, soft_cap=cap, **kw)
+        torch.cuda.synchronize()
+        check(o, l, tag)
+    call = tda.prepare_decode(q, k, v, table, lens_t, scale, soft_cap=cap, kv_split=4, single_launch=True)
+    call.run()
+    torch.cuda.synchronize()
+    check(call.out, call.lse, "single launch")
+    k8, ks, v8, vs, kd, vd = _quantized_two_segment(k, v, dtype)
+    for tag, kw in (("fp8 auto", {}), ("fp8 equal shares", dict(force_balanced=True)), ("fp8 3 chunks", dict(kv_split=3))):
+        o, l = tda.flash_decode(q, k8, v8, table, lens_t, scale, soft_cap=cap, k_scale=ks, v_scale=vs, **kw)
+        torch.cuda.synchronize()
+        assert float(o[1].abs().max()) == 0 and bool((l[1] == -math.inf).all()), tag
+        _check(o[live], l[live], q[live], k8, v8, table[live], [lens[i] for i in live], scale, cap, ref_kv=(kd, vd),
+               tag=f"heads={heads} P={page} {tag}")
+
+
 def _quantized_two_segment(k16, v16, dtype):
     """e4m3 caches with per-kv-head scales from the 16-bit caches of _two_segment_inputs (whose last page holds NaN for
     the unused table columns), and what they dequantise to in ``dtype``."""

@@ -37,6 +37,8 @@ SOURCES = [
     "fdk_splitkv_mfma_d576v512.hip", "fdk_splitkv_mfma_d576v512_queue.hip", "fdk_splitkv_mfma_d576v512_bal.hip",
     # ... large q-head groups on one kv head: the wavefronts of a workgroup share the staged tiles
     "fdk_splitkv_mfma_d576v512_shared.hip", "fdk_splitkv_mfma_d576v512_shared_queue.hip", "fdk_splitkv_mfma_d576v512_shared_bal.hip",
+    # rows of 128 values with more than 16 q heads per kv head
+    "fdk_splitkv_mfma_d128_tiled.hip", "fdk_splitkv_mfma_d128_tiled_queue.hip", "fdk_splitkv_mfma_d128_tiled_bal.hip",
 ]
 
 # the translation units that contain the matrix-core split kernel: the only ones the timeline build compiles anew

@@ -286,11 +286,13 @@ template <int QDT, bool FP8, int PM, int NBUF, int D, bool PROBE = false, int MO
 __global__ __launch_bounds__(512) void splitkv_mfma_kernel(const SplitParams p) {
     constexpr int DK = D, DV = D;
     constexpr bool REUSE = false;
+    constexpr bool kPairedRows = true;
 #include "fdk_splitkv_mfma_body.h"
 #include "fdk_splitkv_mfma_work.h"
 }
 // Rows of two segments and V rows shorter than K rows (q / K rows of DK values, V / output rows of DV): 16-bit and fp8
-// caches, one register buffer.  Beyond 512 values per token and kv head a workgroup has four wavefronts, each alone on its
+// caches, one register buffer.  Also rows of 128 values where a kv head has more than 16 q heads (DK = DV = 128): the
+// q-head tiles of a kv head then run on one XCD and load with plain loads (REUSE), which the kernels above do not.  Beyond 512 values per token and kv head a workgroup has four wavefronts, each alone on its
 // SIMD with the whole register file.
 constexpr int rows2_max_threads(int dk, int dv) { return dk + dv > 512 ? 256 : 512; }
 // REUSE: several workgroups read the same K / V rows (more than one q-head tile per kv head).
@@ -298,6 +300,7 @@ template <int QDT, int PM, int DK, int DV, int MODE, bool REUSE, bool FP8 = fals
 __global__ __launch_bounds__(rows2_max_threads(DK, DV)) void splitkv_mfma_rows2_kernel(const SplitParams p) {
     constexpr bool PROBE = false;
     constexpr int NBUF = 1;
+    constexpr bool kPairedRows = false;
 #include "fdk_splitkv_mfma_body.h"
 #include "fdk_splitkv_mfma_work.h"
 }

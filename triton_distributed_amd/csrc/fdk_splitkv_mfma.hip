@@ -15,6 +15,7 @@ FDK_DECLARE_MFMA(192)            // rows of two segments (128 + 64)
 FDK_DECLARE_MFMA(192v128)        // ... with V rows of 128 values
 FDK_DECLARE_MFMA(576v512)        // 512 + 64, V rows of 512
 FDK_DECLARE_MFMA(576v512_shared) // ... large q-head groups: wavefronts share the staged tiles
+FDK_DECLARE_MFMA(128_tiled)      // rows of 128 values, more than 16 q heads per kv head: q-head tiles on one XCD
 #undef FDK_DECLARE_MFMA
 // (the same rule as mfma_work_mode in the kernel header, which this file does not include)
 static int work_mode_of(const SplitParams& p) {
@@ -94,6 +95,10 @@ int launch_splitkv_mfma(const SplitParams& p, int q_dtype, int kv_dtype, hipStre
             FDK_MFMA_CASE(576v512, 576 * 1024 + 512)
             default: return (int)hipErrorInvalidValue;
         }
+    }
+    // several q-head tiles per kv head read the same rows: the kernels that keep them on one XCD (no single-launch form)
+    if (p.head_dim == 128 && p.group > 16 && !p.fused) {
+        switch (p.head_dim) { FDK_MFMA_CASE(128_tiled, 128) }
     }
     switch (p.head_dim) {
         FDK_MFMA_CASE(64, 64)

@@ -1,6 +1,6 @@
 // The body of the matrix-core split-KV kernels (fdk_splitkv_mfma.h includes this file inside each of its two kernel
-// definitions, which supply: QDT, FP8, PM, NBUF, PROBE, MODE, REUSE, DK = values per q and K row, DV = values per V and
-// output row, and the argument block p).  Kept as text shared by the two kernels rather than as a function they
+// definitions, which supply: QDT, FP8, PM, NBUF, PROBE, MODE, REUSE, kPairedRows, DK = values per q and K row, DV = values
+// per V and output row, and the argument block p).  Kept as text shared by the two kernels rather than as a function they
 // call: the kernel arguments then stay where the compiler reads them with scalar loads.
     constexpr bool BAL = MODE == WM_SHARES;
     using M = Mma<QDT>;
@@ -11,7 +11,8 @@
     // K and V rows alike and of one power-of-two segment (head_dim 64, 128, 256): K and V loads pair up, every load
     // instruction covers the same rows, and all page modes, fp8 caches, two register buffers and the single-launch
     // form are built.  Otherwise (192, 576 / 512 ...): one buffer, page numbers per tile or per row.
-    constexpr bool kOneSegment = DK == DV && RK::D1 == 0;
+    // (kPairedRows, from the kernel definition: false in the kernels that take every row length through the general code)
+    constexpr bool kOneSegment = kPairedRows && DK == DV && RK::D1 == 0;
     // One-byte rows of 192 values are one and a half 128-byte lines: neighbouring kv heads of a token share a line, and
     // workgroups with an odd number of kv heads are mapped so that those neighbours run on one XCD (one L2 fetches the
     // line once; spread over the XCDs in dispatch order every head's L2 fetched both of its partial lines).
