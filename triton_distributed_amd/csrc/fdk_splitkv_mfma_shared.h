@@ -39,6 +39,19 @@ namespace fdk {
 
 namespace {
 
+// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 without the LDS crossbar: v_permlane16_swap exchanges the odd rows (16
+// lanes) of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the lower
+// half of the second; applied to two copies of x they leave (x[l & ~16], x[l | 16]) resp. (x[l & 31], x[l | 32]) in lane l.
+// (From inline asm: given the same value twice, the compiler folds the builtins' two results into one.)
+__device__ __forceinline__ float max_across_rows(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    a = fmaxf(a, b);
+    b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 constexpr int kSharedWaves = 8;                        // wavefronts per workgroup
 constexpr int kSharedColSplit = 2;                     // wavefronts that share a tile of 16 q heads, each with 1 / kSharedColSplit
                                                        // of the output columns (both form the tile's logits and softmax)
@@ -546,9 +559,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 for (int i = 0; i < 4; ++i)
                     if (tok0 + 4 * a + i >= c_end) sv[i] = -INFINITY;
             }
-            float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));          // finite: token tok0 is valid
+            const float mx = max_across_rows(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));     // finite: token tok0 is valid
             if (__builtin_amdgcn_ballot_w64(mx > m_ref + kSlack) != 0) {
                 mx_seen = mx;
                 return false;
