@@ -277,6 +277,19 @@ __device__ __forceinline__ void tiles_on_one_xcd(int id, int rows, int T, int& r
     }
 }
 
+// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 without the LDS crossbar: v_permlane16_swap exchanges the odd rows (16
+// lanes) of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the lower
+// half of the second; applied to two copies of x they leave (x[l & ~16], x[l | 16]) resp. (x[l & 31], x[l | 32]) in lane l.
+// (From inline asm: given the same value twice, the compiler folds the builtins' two results into one.)
+__device__ __forceinline__ float max_across_rows(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    a = fmaxf(a, b);
+    b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 // Eight wavefronts may share a kv head where a tile is small: one-byte caches with rows of 192 values (6 KB a tile;
 // four wavefronts would keep 24 KB of a compute unit under way, eight keep 48 KB).
 constexpr bool rows2_eight_share(bool fp8, int dk, int dv) { return fp8 && dk + dv <= 384; }

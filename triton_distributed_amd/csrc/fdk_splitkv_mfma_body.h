@@ -422,8 +422,14 @@
                 if (tok0 + 4 * a + i >= c_end) sv[i] = -INFINITY;
         }
         float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));          // finite: token tok0 is valid
+        // (finite: token tok0 is valid.  Without the LDS crossbar where the vector ALU and the LDS are what a kernel waits
+        // for - one-byte caches, the general row code; the 16-bit one-segment kernels wait for memory and stay as they are)
+        if constexpr (FP8 || !kPairedRows) {
+            mx = max_across_rows(mx);
+        } else {
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        }
         const float m_new = fmaxf(m_run, mx);
         const float alpha = fast_exp2(m_run - m_new);
         float pr[4];

@@ -39,19 +39,6 @@ namespace fdk {
 
 namespace {
 
-// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 without the LDS crossbar: v_permlane16_swap exchanges the odd rows (16
-// lanes) of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the lower
-// half of the second; applied to two copies of x they leave (x[l & ~16], x[l | 16]) resp. (x[l & 31], x[l | 32]) in lane l.
-// (From inline asm: given the same value twice, the compiler folds the builtins' two results into one.)
-__device__ __forceinline__ float max_across_rows(float x) {
-    float a = x, b = x;
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    a = fmaxf(a, b);
-    b = a;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    return fmaxf(a, b);
-}
-
 constexpr int kSharedWaves = 8;                        // wavefronts per workgroup
 constexpr int kSharedColSplit = 2;                     // wavefronts that share a tile of 16 q heads, each with 1 / kSharedColSplit
                                                        // of the output columns (both form the tile's logits and softmax)
