@@ -214,6 +214,19 @@ def bench_kv_append(args):
     }), flush=True)
 
 
+def _split_kernel_name(cfg, plan):
+    """The kernel family that the library runs this configuration in (the rule of mfma_heads_per_wg and of the dispatch in
+    csrc/fdk_splitkv_mfma.hip): the name under which rocprofv3 lists the split kernel."""
+    if plan.algo != "mfma":
+        return f"splitkv_{plan.algo}_kernel"
+    dk, dv, group, fp8 = cfg.head_dim, cfg.dv, cfg.q_heads // cfg.kv_heads, cfg.kv_dtype == "fp8_e4m3"
+    if dk + dv > 512 and (not fp8 or group > 16):
+        return "splitkv_mfma_shared_kernel"
+    if dk != dv or dk == 192 or (dk == 128 and group > 16):
+        return "splitkv_mfma_rows2_kernel"
+    return "splitkv_mfma_kernel"
+
+
 def _time_launches(torch, fn, n_iter, warm=10):
     """Average microseconds per call of fn(i), HIP events on the current stream around n_iter back-to-back calls."""
     for i in range(warm):
@@ -790,7 +803,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": f"splitkv_{plan.algo}_kernel",
+            "kernel": _split_kernel_name(inp.cfg, plan),
             "variant": "single pass: writes (out, lse) itself" if single_pass else "writes fp32 partials; the combine kernel follows",
             "achieved": round(split_gbps, 1),
             "peak": HBM_PEAK_GBPS,
