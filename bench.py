@@ -69,6 +69,9 @@ def parse_args():
     ap.add_argument("--fp8-fold", action="store_true",
                     help="fp8 cache: apply the K scale to the logits instead of to every K value "
                          "(FDK_FLAG_FP8_FOLD_K_SCALE; off the dequantise-then-decode definition by the 16-bit rounding of K)")
+    ap.add_argument("--fp8-pow2-scales", action="store_true",
+                    help="fp8 cache: round the per-kv-head scales up to powers of two (as an unscaled cache has them: 1.0); "
+                         "the library then applies the K scale as the exponent operand of the conversion, which is exact")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the prepared calls only: no legs on other pools, no graph replay, no un-prepared or "
                          "reference-named entry points, no CPU baseline - for profiler runs, so that every dispatch of a "
@@ -533,6 +536,9 @@ def main():
     inp_cpu = wl.make_inputs(_config_of(args, wl))
     print(f"[bench] generated {args.config} on CPU in {time.perf_counter() - t_gen:.1f}s", file=sys.stderr, flush=True)
     inp = inp_cpu.to(dev)
+    if args.fp8_pow2_scales and inp.cfg.kv_dtype == "fp8_e4m3":      # (timing only: the cache keeps its codes)
+        inp.k_scale = torch.exp2(torch.ceil(torch.log2(inp.k_scale)))
+        inp.v_scale = torch.exp2(torch.ceil(torch.log2(inp.v_scale)))
     pools = [(inp.k_cache, inp.v_cache)]
     pool_bytes = (inp.k_cache.numel() + inp.v_cache.numel()) * inp.k_cache.element_size()
     rotate = max(1, args.rotate)
@@ -793,7 +799,9 @@ def main():
             "balanced": plan.balanced, "workgroups": plan.workgroups, "kv_heads_per_wg": plan.kv_heads_per_wg,
             "single_launch": bool(args.single_launch and plan.num_splits > 1),
             "fp8_k_scale": None if inp.cfg.kv_dtype != "fp8_e4m3" else
-                           ("folded into the logit scale" if args.fp8_fold else "applied to every K value (exact dequantisation)"),
+                           ("folded into the logit scale" if args.fp8_fold else
+                            "powers of two: the exponent operand of the conversion (exact dequantisation)" if args.fp8_pow2_scales else
+                            "applied to every K value (exact dequantisation)"),
             "kv_pool_placement": ("one allocation per (K, V) pair, V 256 bytes off K modulo 512 (alloc_kv_pools, as PagedKVCache "
                                   "allocates)" if args.kv_placement == "staggered" else "two independent torch allocations"),
             "kv_pools_rotated": len(pools), "forced_kv_split": args.kv_split if args.kv_split > 0 else None,

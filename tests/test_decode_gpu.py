@@ -1855,6 +1855,37 @@ def test_fp8_every_byte_value_dequantises_exactly(cuda_device, algo):
     assert torch.equal(out[:, 0, 0], want) and torch.equal(out[:, 0, 127], want)
 
 
+@pytest.mark.parametrize("dims,heads", [((128, 128), (4, 1)), ((192, 128), (4, 2)), ((576, 512), (4, 1)), ((576, 512), (40, 1))])
+@pytest.mark.parametrize("k_scale", [1.0, 0.5, 2.0 ** -7, 8.0, 0.75])
+def test_fp8_k_scales_that_are_powers_of_two(cuda_device, dims, heads, k_scale):
+    """A K scale that is a power of two goes into the conversion instruction as an exponent instead of a multiplication per
+    value: the logit of a one-hot query over a single token is the dequantised K value, for every e4m3 code, in every
+    kernel family (one-segment, two-segment, shared tiles); 0.75 takes the multiplications, as a control."""
+    dk, dv = dims
+    hq, hkv = heads
+    table = torch.from_numpy(ofp8.e4m3fn_table())
+    codes = torch.tensor([c for c in range(256) if not math.isnan(table[c])], dtype=torch.uint8)
+    n = codes.numel()
+    # sequence i: one token whose K row holds code i everywhere; q head h is one-hot at column 37 h + 5
+    k8 = codes.view(n, 1, 1, 1).expand(n, 1, hkv, dk).contiguous().view(torch.float8_e4m3fn).to(cuda_device)
+    v8 = torch.zeros(n, 1, hkv, dv, dtype=torch.uint8).view(torch.float8_e4m3fn).to(cuda_device)
+    q = torch.zeros(n, hq, dk, dtype=torch.bfloat16)
+    for h in range(hq):
+        q[:, h, (37 * h + 5) % dk] = 1.0
+    q = q.to(cuda_device)
+    ks = torch.full((hkv,), k_scale, device=cuda_device)
+    vs = torch.ones(hkv, device=cuda_device)
+    bt = torch.arange(n, dtype=torch.int32, device=cuda_device)[:, None].contiguous()
+    sm = 0.125
+    out, lse = tda.flash_decode(q, k8, v8, bt, _lens_t([1] * n, cuda_device), sm, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    want = (table[codes.long()].double() * k_scale).to(torch.bfloat16).double() * sm       # (exact in bf16 for powers of two)
+    got = lse.double().cpu()
+    assert float(out.abs().max()) == 0
+    for h in (0, hq - 1):
+        torch.testing.assert_close(got[:, h], want, atol=2e-6, rtol=2e-6, msg=lambda m: f"dims={dims} k_scale={k_scale} head {h}: {m}")
+
+
 # ---- the five benchmark configurations at full size ----------------------------------------------------------------
 _INPUT_CACHE = {}
 

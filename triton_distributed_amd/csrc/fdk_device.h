@@ -168,6 +168,12 @@ __device__ __forceinline__ uint4 load_stream16(const void* p) {
     return make_uint4(x.x, x.y, x.z, x.w);
 }
 
+// Whether an fp8 dequantisation scale is a power of two within 2^-40 .. 2^40 (1.0, the usual value of an unscaled cache,
+// among them): then k8 * scale is exactly what the conversion instruction gives with the scale as its exponent operand.
+__device__ __forceinline__ bool is_pow2_scale(float s) {
+    const uint32_t b = __builtin_bit_cast(uint32_t, s);
+    return (b & 0x007fffffu) == 0 && (b >> 23) >= 127u - 40u && (b >> 23) <= 127u + 40u;
+}
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
@@ -291,6 +297,11 @@ template <> struct Pack2<FDK_BF16> {
         return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, 1.0f, true)
                                                : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, 1.0f, false));
     }
+    // ... times 2^e, e the exponent of `pow2` (a power of two): still exact, e4m3 values have four significant bits
+    static __device__ __forceinline__ uint32_t from_fp8(uint32_t four, bool hi, float pow2) {
+        return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, pow2, true)
+                                               : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(four, pow2, false));
+    }
 };
 template <> struct Pack2<FDK_FP16> {
     using vec = f16x2_t;
@@ -306,6 +317,10 @@ template <> struct Pack2<FDK_FP16> {
     static __device__ __forceinline__ uint32_t from_fp8(uint32_t four, bool hi) {
         return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, 1.0f, true)
                                                : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, 1.0f, false));
+    }
+    static __device__ __forceinline__ uint32_t from_fp8(uint32_t four, bool hi, float pow2) {
+        return __builtin_bit_cast(uint32_t, hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, pow2, true)
+                                               : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(four, pow2, false));
     }
 };
 

@@ -156,9 +156,13 @@
     // four values.  Folded (p.fp8_fold): the values are converted exactly (two instructions per four values) and the
     // head's scale multiplies the logits - (q . k8) * scale instead of q . round(k8 * scale), which differs by the
     // rounding of K to the 16-bit type (relative 2^-9 per element).
-    const bool fold = FP8 && p.fp8_fold;
-    const float logit_scale_log2 = fold ? p.scale_log2 * kscale : p.scale_log2;
-    const float logit_scale = fold ? p.sm_scale * kscale : p.sm_scale;
+    // (A scale that is a power of two needs neither: the conversion instruction applies it as an exponent, which is the
+    // exact k8 * scale - the code of the folded form with the scale in the conversion instead of in the logit scale.)
+    const bool by_exponent = FP8 && !p.fp8_fold && is_pow2_scale(kscale);
+    const bool fold = FP8 && (p.fp8_fold || by_exponent);
+    const float kconv = by_exponent ? kscale : 1.0f;      // the scale operand of the K conversions of the folded form
+    const float logit_scale_log2 = fold && !by_exponent ? p.scale_log2 * kscale : p.scale_log2;
+    const float logit_scale = fold && !by_exponent ? p.sm_scale * kscale : p.sm_scale;
 
     const char* kbase = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES + lpiece * 16;
     const char* vbase = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES + lpiece * 16;
@@ -297,8 +301,8 @@
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     if (fold) {
-                        o[2 * w] = P2::from_fp8(in[w], false);
-                        o[2 * w + 1] = P2::from_fp8(in[w], true);
+                        o[2 * w] = P2::from_fp8(in[w], false, kconv);
+                        o[2 * w + 1] = P2::from_fp8(in[w], true, kconv);
                     } else {
                         const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(in[w], false);
                         const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(in[w], true);
@@ -337,8 +341,8 @@
                 if (fold) {
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        ko[2 * w] = P2::from_fp8(rg.k[j][w], false);
-                        ko[2 * w + 1] = P2::from_fp8(rg.k[j][w], true);
+                        ko[2 * w] = P2::from_fp8(rg.k[j][w], false, kconv);
+                        ko[2 * w + 1] = P2::from_fp8(rg.k[j][w], true, kconv);
                     }
                 } else {
 #pragma unroll

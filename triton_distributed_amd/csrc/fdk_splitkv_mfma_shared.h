@@ -168,9 +168,13 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             if (p.k_scale) kscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.k_scale))[kvh]);
             if (p.v_scale) vscale = __builtin_bit_cast(float, as_const(reinterpret_cast<const int32_t*>(p.v_scale))[kvh]);
         }
-        const bool fold = FP8 && p.fp8_fold;
-        const float logit_scale_log2 = fold ? p.scale_log2 * kscale : p.scale_log2;
-        const float logit_scale = fold ? p.sm_scale * kscale : p.sm_scale;
+        // (A scale that is a power of two needs neither: the conversion instruction applies it as an exponent, which is the
+        // exact k8 * scale - the code of the folded form with the scale in the conversion instead of in the logit scale.)
+        const bool by_exponent = FP8 && !p.fp8_fold && is_pow2_scale(kscale);
+        const bool fold = FP8 && (p.fp8_fold || by_exponent);
+        const float kconv = by_exponent ? kscale : 1.0f;      // the scale operand of the K conversions of the folded form
+        const float logit_scale_log2 = fold && !by_exponent ? p.scale_log2 * kscale : p.scale_log2;
+        const float logit_scale = fold && !by_exponent ? p.sm_scale * kscale : p.sm_scale;
         const char* kplane = reinterpret_cast<const char*>(p.k) + ((int64_t)kvh * p.k_sh) * ES;
         const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
         const uint32_t ksp_bytes = (uint32_t)(p.k_sp * ES), vsp_bytes = (uint32_t)(p.v_sp * ES);
@@ -365,8 +369,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
                         if (fold) {
-                            o[2 * w] = P2::from_fp8(r[w], false);
-                            o[2 * w + 1] = P2::from_fp8(r[w], true);
+                            o[2 * w] = P2::from_fp8(r[w], false, kconv);
+                            o[2 * w + 1] = P2::from_fp8(r[w], true, kconv);
                         } else {
                             const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], false);
                             const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], true);
