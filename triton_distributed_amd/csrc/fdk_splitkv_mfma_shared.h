@@ -72,10 +72,15 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     // first segments instead of behind each row, and the swizzle is applied on the memory side: the lane whose bytes
     // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).  e4m3 caches pass
     // through registers for the conversion (two staged tiles).
-    constexpr bool kDirect = !FP8;
-    constexpr int kStaged = kDirect ? 4 : 2;   // staged tiles in LDS
-    static_assert(!kDirect || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
+    // e4m3 caches with page numbers per tile (kRaw): the bytes take the same road into one of two raw tiles in LDS, and
+    // the wavefront that requested them converts them from there into a staged tile (its own share only: no other
+    // wavefront has to know when they landed); three staged tiles.  With page numbers per row they pass through registers.
+    constexpr bool kRaw = FP8 && PM == PM_TILE;
+    constexpr bool kDirect = !FP8 || kRaw;
+    constexpr int kStaged = kRaw ? 3 : kDirect ? 4 : 2;   // staged tiles in LDS
+    static_assert(!kDirect || kRaw || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
                   "direct loads: a first segment of 1 KB per row, a second K segment of 128 bytes");
+    static_assert(!kRaw || (RK::NJ0 == NW && RV::NJ0 == NW && RK::NJ1 == 1 && RV::D1 == 0), "raw tiles: rows of 512 (+ 64) one-byte values");
     constexpr int kK0Row = kDirect ? RK::D0 * 2 : RBK;                 // bytes from one staged row's first K segment to the next row's
     constexpr int kK1Base = kDirect ? kTile * RK::D0 * 2 : RK::D0 * 2; // where row 0's second K segment starts, and
     constexpr int kK1Row = kDirect ? RK::D1 * 2 : RBK;                 // the step to the next row's
@@ -259,6 +264,100 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 const int j = slot_instr(s, RV::NJ0);
                 const uint32_t byte = (uint32_t)((ln ^ ((j & 3) << 1)) << 4);
                 load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j, 0, byte, byte, vplane, vsp_bytes, vst_bytes), dst + kTile * RBK + j * 1024);
+            }
+        };
+        // ---- e4m3 rows through raw tiles (kRaw).  The load instructions and their lanes are those of the register path
+        // (issue): instruction j of a segment covers rows j RPL .., 16 bytes per lane; it fills 1 KB of the raw tile, first K
+        // segments, second K segment, V rows.  convert_raw reads back exactly the bytes this wavefront requested. ----
+        // Two raw tiles of first K segments and V rows, each wavefront reading back only what it requested itself; the
+        // second K segment, one instruction that every wavefront issues and converts alike (so that all issue the same
+        // number of loads), has four places of its own: a wavefront requests tile t + 4's into the place of tile t's, which
+        // every wavefront converted two barriers ago - with two places a fast wavefront would overwrite what a slow one has
+        // yet to read.
+        constexpr int kRawTile = (RK::NJ0 + RV::NJ0) * 1024;
+        const uint32_t raw_lds = (uint32_t)(kStaged * kTileBytes + 16 + 2 * NW * 1024);      // offset of the raw tiles from lds[0]
+        const uint32_t raw1_lds = raw_lds + 2 * kRawTile;                                    // ... and of the second K segments
+        auto issue_raw = [&](auto clamp_tag, int t, int32_t pg_id) {
+            const int tok0 = c_start + t * kTile;
+            const uint32_t dst = lds0 + raw_lds + (uint32_t)(t & 1) * kRawTile;
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            ln &= 63;
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j * RK::RPL0, ln / RK::LPR0, k_lane0, (ln % RK::LPR0) * 16, kplane,
+                                      ksp_bytes, kst_bytes), dst + j * 1024);
+            }
+#pragma unroll
+            for (int s = 0; s < KS1; ++s) {
+                const int j = slot_instr(s, RK::NJ1);
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j * RK::RPL1, ln / RK::LPR1, k_lane1, RK::D0 * ES + (ln % RK::LPR1) * 16,
+                                      kplane, ksp_bytes, kst_bytes), lds0 + raw1_lds + (uint32_t)(t & 3) * (RK::NJ1 * 1024) + j * 1024);
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j * RV::RPL0, ln / RV::LPR0, v_lane0, (ln % RV::LPR0) * 16, vplane,
+                                      vsp_bytes, vst_bytes), dst + (RK::NJ0 + j) * 1024);
+            }
+        };
+        // 16 one-byte values -> two 16-byte chunks of 16-bit values (K: times the head's scale, see above; V: exact)
+        auto widen = [&](const uint4 in, auto is_k, uint4& lo, uint4& hi) {
+            constexpr bool K = decltype(is_k)::value;
+            const uint32_t r[4] = {in.x, in.y, in.z, in.w};
+            uint32_t o[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                if (!K) {
+                    o[2 * w] = P2::from_fp8(r[w], false);
+                    o[2 * w + 1] = P2::from_fp8(r[w], true);
+                } else if (fold) {
+                    o[2 * w] = P2::from_fp8(r[w], false, kconv);
+                    o[2 * w + 1] = P2::from_fp8(r[w], true, kconv);
+                } else {
+                    const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], false);
+                    const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], true);
+                    o[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
+                    o[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
+                }
+            }
+            lo = make_uint4(o[0], o[1], o[2], o[3]);
+            hi = make_uint4(o[4], o[5], o[6], o[7]);
+        };
+        auto convert_raw = [&](int t, char* buf) {
+            const char* raw = lds + raw_lds + (t & 1) * kRawTile;
+            const char* raw1 = lds + raw1_lds + (t & 3) * (RK::NJ1 * 1024);
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            ln &= 63;
+            uint4 lo, hi;
+#pragma unroll
+            for (int s = 0; s < KS0; ++s) {
+                const int j = slot_instr(s, RK::NJ0);
+                const int row = j * RK::RPL0 + ln / RK::LPR0, piece = ln % RK::LPR0;
+                widen(*reinterpret_cast<const uint4*>(raw + j * 1024 + ln * 16), BoolTag<true>(), lo, hi);
+                char* at = buf + row * kK0Row;
+                *reinterpret_cast<uint4*>(at + (((2 * piece) ^ (row & 7)) << 4)) = lo;
+                *reinterpret_cast<uint4*>(at + (((2 * piece + 1) ^ (row & 7)) << 4)) = hi;
+            }
+#pragma unroll
+            for (int s = 0; s < KS1; ++s) {
+                const int j = slot_instr(s, RK::NJ1);
+                const int row = j * RK::RPL1 + ln / RK::LPR1, piece = ln % RK::LPR1;
+                widen(*reinterpret_cast<const uint4*>(raw1 + j * 1024 + ln * 16), BoolTag<true>(), lo, hi);
+                char* at = buf + kK1Base + row * kK1Row;
+                *reinterpret_cast<uint4*>(at + (((2 * piece) ^ (row & 7)) << 4)) = lo;
+                *reinterpret_cast<uint4*>(at + (((2 * piece + 1) ^ (row & 7)) << 4)) = hi;
+            }
+#pragma unroll
+            for (int s = 0; s < VS0; ++s) {
+                const int j = slot_instr(s, RV::NJ0);
+                const int row = j * RV::RPL0 + ln / RV::LPR0, piece = ln % RV::LPR0;
+                widen(*reinterpret_cast<const uint4*>(raw + (RK::NJ0 + j) * 1024 + ln * 16), BoolTag<false>(), lo, hi);
+                char* lv = buf + kTile * RBK;
+                *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, 2 * piece)) = lo;
+                *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, 2 * piece + 1)) = hi;
             }
         };
         // Page numbers per row (PM_ROW) for the direct loads.  A vector load that the compiler sees would make it wait, in
@@ -600,10 +699,13 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // under way" otherwise.  (Loads that the compiler sees - page numbers per row, PM_ROW - only make these waits,
             // and the compiler's own, wait for more than they need.)
             const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
-            auto staged = [&](int t) { return lds + (t & 3) * kTileBytes; };
+            auto staged = [&](int t) { return lds + (t % kStaged) * kTileBytes; };
             auto issue_tile = [&](int t, int32_t pg_id) {
-                const uint32_t dst = lds0 + (uint32_t)(t & 3) * kTileBytes;
-                if (PM == PM_ROW) {
+                const uint32_t dst = lds0 + (uint32_t)(t % kStaged) * kTileBytes;
+                if constexpr (kRaw) {
+                    if (t < n_full) issue_raw(BoolTag<false>(), t, pg_id);
+                    else if (t < n_tiles) issue_raw(BoolTag<true>(), t, pg_id);
+                } else if (PM == PM_ROW) {
                     if (t < n_tiles) issue_direct_rows(t, dst);
                 } else if (t < n_full) {
                     issue_direct(BoolTag<false>(), t, pg_id, dst);
@@ -614,7 +716,24 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // the staged tiles are free: no wavefront still reads the previous piece's, none of its loads is under way
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
             int32_t pg_hold = 0;
-            if (PM == PM_ROW) {
+            // kRaw: one round of a tile's bytes - wait until this wavefront's share of tile u has landed in its raw tile (its
+            // loads return in order: all but those of tile u + 1), convert it into the staged tile, request tile u + 2 into
+            // the raw tile just read.
+            auto advance_raw = [&](int u) {
+                if (u + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerTile) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                if (u < n_tiles) convert_raw(u, staged(u));
+                const int32_t pg_now = pg_hold;
+                pg_hold = page_id(u + 3);
+                issue_tile(u + 2, pg_now);
+            };
+            if constexpr (kRaw) {
+                issue_tile(0, page_id(0));
+                issue_tile(1, page_id(1));
+                pg_hold = page_id(2);
+                advance_raw(0);
+                advance_raw(1);
+            } else if (PM == PM_ROW) {
                 // page numbers per row come through LDS as well (issue_pages), two steps ahead of the rows that need them
 #pragma unroll
                 for (int t = 0; t < 5; ++t) issue_pages(t);
@@ -634,15 +753,20 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // tiles ahead are loads it does not know of.  (An empty asm that takes the registers as operands is such a use.)
 #pragma unroll
             for (int i = 0; i < KQ; ++i) asm volatile("" : "+v"(qreg[i].x), "+v"(qreg[i].y), "+v"(qreg[i].z), "+v"(qreg[i].w));
-            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");          // tile 0 is there
-            static_assert(kLoadsPerTile == 5, "the waits below count the loads of one tile");
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");          // tile 0 is there
+            static_assert(kLoadsPerTile == (kRaw ? 3 : 5), "the waits below count the loads of one tile");
             // (the barrier also waits for this wavefront's LDS operations: its half of the next tile's dot products is in
             // the exchange area, its reads of the partner's half of the tile before are done)
             // PM_ROW: a step requests the rows of tile t + 3 and then the page numbers of tile t + 5, one load more; what has
             // to have landed at the top of step t are the rows of tile t + 1 and the page numbers of tile t + 3, both requested
             // in step t - 2: everything but the loads of step t - 1, which are six, or the one of the page numbers alone.
             auto step = [&](int t) {
-                if (PM == PM_ROW) {
+                if constexpr (kRaw) {
+                    // (every wavefront has converted its share of tile t + 1 and is done with tile t - 1, whose staged tile
+                    // takes tile t + 2)
+                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    advance_raw(t + 2);
+                } else if (PM == PM_ROW) {
                     if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                     else asm volatile("s_waitcnt vmcnt(1) lgkmcnt(0)\n\ts_barrier" ::: "memory");
                     issue_tile(t + 3, 0);
@@ -787,8 +911,10 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
     p.hg_blocks = p.hkv;
     // staged tiles, the next work item, and (direct loads) the exchange area of the half dot products: see kDirect
-    const size_t lds_bytes = FP8 ? 2 * (size_t)kTileBytes + 16 : 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 8 * 256;   // (+ page numbers)
     const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
+    const size_t lds_bytes = !FP8 ? 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 8 * 256      // (+ page numbers)
+                           : pm == PM_TILE ? 3 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 2 * 16384 + 4 * 1024   // (+ raw tiles)
+                                           : 2 * (size_t)kTileBytes + 16;
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
     // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
     // than there are pieces: every workgroup of the queue has to take one, or it would not be counted among the
