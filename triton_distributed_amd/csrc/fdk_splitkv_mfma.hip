@@ -43,8 +43,8 @@ bool mfma_supported(int q_dtype, int kv_dtype, int /*group*/, int head_dim, int 
 // load and stage every tile once for four tiles of 16 q heads.  16-bit caches: whatever the group, the rows of those
 // kernels go straight from memory into LDS, which beats the 16-head kernels even where most of a workgroup's wavefronts
 // have no q heads and only help to load (batch 32 x 4096 tokens, 8 / 16 / 32 q heads: 51 / 52 / 56 us against 75 / 77 /
-// 115 us).  e4m3 caches pass through registers either way: from 17 q heads on (8 / 16 / 32 q heads: 58 / 59 / 66 us
-// against 50 / 52 / 90 us).
+// 115 us).  e4m3 caches, whose values have to be converted on the way: from 17 q heads on (8 / 16 / 32 q heads: 52 / 53 /
+// 58 us against 50 / 52 / 90 us).
 int mfma_heads_per_wg(int group, int row_values, int kv_dtype) {
     return row_values > 512 && (kv_dtype != FDK_FP8_E4M3 || group > 16) ? 64 : 16;
 }

@@ -27,10 +27,13 @@
 // head tile also split the q . k products - even and odd k-steps, nine each, 36 registers of Q^T each - and exchange
 // their halves through LDS; a step of the loop holds the half dot products of tile t + 1 next to the softmax and the PV
 // product of tile t, which do not depend on each other, and ONE barrier.
-// e4m3 caches: the rows pass through registers for the conversion (each wavefront loads its share two tiles ahead and
-// stores it, converted, into one of two staged tiles; one barrier per tile: a wavefront writes tile t + 1 only after
-// the barrier of tile t, which every wavefront reaches after it has finished reading tile t - 1 from the same buffer);
-// every wavefront forms all of its head tile's dot products (six interleaved accumulation chains, Q^T in 72 registers).
+// e4m3 caches, page numbers per tile (kRaw): the bytes take the same road into one of two raw tiles in LDS, and the
+// wavefront that requested them converts its own share from there into one of three staged tiles; the steps are those
+// of the 16-bit kernels.  Page numbers per row: the rows pass through registers (each wavefront loads its share two tiles
+// ahead and stores it, converted, into one of two staged tiles; one barrier per tile: a wavefront writes tile t + 1 only
+// after the barrier of tile t, which every wavefront reaches after it has finished reading tile t - 1 from the same
+// buffer); every wavefront forms all of its head tile's dot products (six interleaved accumulation chains, Q^T in 72
+// registers).
 #pragma once
 
 #include "fdk_splitkv_mfma.h"
