@@ -18,22 +18,18 @@
 // the output tile (see move_reference).  Page numbers per tile or per row (PM_TILE, PM_ROW).  How pieces are handed out
 // is shared with the other kernels (fdk_splitkv_mfma_work.h) with a head tile of 64 q heads.
 //
-// 16-bit caches (kDirect): the rows never pass through registers.  global_load_lds_dwordx4 writes the 16 bytes of lane i
-// to LDS byte M0 + 16 i, so a load instruction fills 1 KB of a staged tile directly; the swizzle of the staged rows is
-// applied on the memory side (the lane whose bytes land in chunk x of row r fetches chunk x ^ swizzle(r) of that row).
-// Four staged tiles: tile t is worked on while tiles t + 1 ... t + 3 land.  The compiler would put "wait for every load
-// under way" in front of each LDS read that follows such a load, so the loads are issued from inline asm and the tile
-// loop waits by count itself (loads return in order, every wavefront issues five per tile).  The two wavefronts of a
-// head tile also split the q . k products - even and odd k-steps, nine each, 36 registers of Q^T each - and exchange
-// their halves through LDS; a step of the loop holds the half dot products of tile t + 1 next to the softmax and the PV
-// product of tile t, which do not depend on each other, and ONE barrier.
-// e4m3 caches, page numbers per tile (kRaw): the bytes take the same road into one of two raw tiles in LDS, and the
-// wavefront that requested them converts its own share from there into one of three staged tiles; the steps are those
-// of the 16-bit kernels.  Page numbers per row: the rows pass through registers (each wavefront loads its share two tiles
-// ahead and stores it, converted, into one of two staged tiles; one barrier per tile: a wavefront writes tile t + 1 only
-// after the barrier of tile t, which every wavefront reaches after it has finished reading tile t - 1 from the same
-// buffer); every wavefront forms all of its head tile's dot products (six interleaved accumulation chains, Q^T in 72
-// registers).
+// The rows never pass through registers.  global_load_lds_dwordx4 writes the 16 bytes of lane i to LDS byte M0 + 16 i, so
+// a load instruction fills 1 KB of LDS directly.  The compiler would put "wait for every load under way" in front of each
+// LDS read that follows such a load, so the loads are issued from inline asm and the tile loop waits by count itself
+// (loads return in order, every wavefront issues the same number per tile).
+// 16-bit caches: the loads fill the staged tile itself; the swizzle of the staged rows is applied on the memory side (the
+// lane whose bytes land in chunk x of row r fetches chunk x ^ swizzle(r) of that row).  Four staged tiles: tile t is
+// worked on while tiles t + 1 ... t + 3 land.
+// e4m3 caches (kRaw): the loads fill one of two raw tiles, and the wavefront that requested them converts its own share
+// from there into one of three staged tiles (16-bit values either way).
+// The two wavefronts of a head tile split the q . k products - even and odd k-steps, nine each, 36 registers of Q^T each -
+// and exchange their halves through LDS; a step of the loop holds the half dot products of tile t + 1 next to the softmax
+// and the PV product of tile t, which do not depend on each other, and ONE barrier.
 #pragma once
 
 #include "fdk_splitkv_mfma.h"
@@ -61,7 +57,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     constexpr bool kOneSegment = false;        // (fdk_splitkv_mfma_work.h: several head tiles of a kv head go to one XCD)
     constexpr bool kRowsShareLines = false;    // (16-bit rows: whole 128-byte lines per kv head)
     constexpr int kTileHeads = kSharedTileHeads;
-    constexpr bool kFirstPieceStraight = !FP8;  // (fdk_splitkv_mfma_work.h; e4m3: one copy of the piece, which needs every register)
+    constexpr bool kFirstPieceStraight = true;  // (fdk_splitkv_mfma_work.h)
     constexpr int NW = kSharedWaves;
     constexpr int ES = FP8 ? 1 : 2;            // bytes per cache value
     constexpr int RBK = 2 * DK, RBV = 2 * DV;  // bytes of a staged row
@@ -73,25 +69,23 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
     // instruction writes its 16 bytes at M0 + 16 i, no registers in between and nothing to store), four staged tiles.
     // A load instruction then fills 1 KB of consecutive LDS, so the second K segment of the 16 rows lies behind their
     // first segments instead of behind each row, and the swizzle is applied on the memory side: the lane whose bytes
-    // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).  e4m3 caches pass
-    // through registers for the conversion (two staged tiles).
-    // e4m3 caches with page numbers per tile (kRaw): the bytes take the same road into one of two raw tiles in LDS, and
-    // the wavefront that requested them converts them from there into a staged tile (its own share only: no other
-    // wavefront has to know when they landed); three staged tiles.  With page numbers per row they pass through registers.
-    constexpr bool kRaw = FP8 && PM == PM_TILE;
-    constexpr bool kDirect = !FP8 || kRaw;
-    constexpr int kStaged = kRaw ? 3 : kDirect ? 4 : 2;   // staged tiles in LDS
-    static_assert(!kDirect || kRaw || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
+    // land in chunk x of row r fetches chunk x ^ swizzle(r) (the same 128-byte line either way).
+    // e4m3 caches (kRaw): the bytes take the same road into one of two raw tiles in LDS, and the wavefront that requested
+    // them converts them from there into a staged tile (its own share only: no other wavefront has to know when they
+    // landed); three staged tiles.
+    constexpr bool kRaw = FP8;
+    constexpr int kStaged = kRaw ? 3 : 4;      // staged tiles in LDS
+    static_assert(kRaw || (RK::LPR0 == 64 && RV::LPR0 == 64 && RV::D1 == 0 && (RK::D1 == 0 || RK::LPR1 == 8)),
                   "direct loads: a first segment of 1 KB per row, a second K segment of 128 bytes");
     static_assert(!kRaw || (RK::NJ0 == NW && RV::NJ0 == NW && RK::NJ1 == 1 && RV::D1 == 0), "raw tiles: rows of 512 (+ 64) one-byte values");
-    constexpr int kK0Row = kDirect ? RK::D0 * 2 : RBK;                 // bytes from one staged row's first K segment to the next row's
-    constexpr int kK1Base = kDirect ? kTile * RK::D0 * 2 : RK::D0 * 2; // where row 0's second K segment starts, and
-    constexpr int kK1Row = kDirect ? RK::D1 * 2 : RBK;                 // the step to the next row's
+    constexpr int kK0Row = RK::D0 * 2;         // bytes from one staged row's first K segment to the next row's
+    constexpr int kK1Base = kTile * RK::D0 * 2; // where row 0's second K segment starts, and
+    constexpr int kK1Row = RK::D1 * 2;         // the step to the next row's
     // load instructions of a tile that one wavefront issues, per segment of the rows (Rows<>)
     constexpr int KS0 = (RK::NJ0 + NW - 1) / NW, KS1 = (RK::NJ1 + NW - 1) / NW;
     constexpr int VS0 = (RV::NJ0 + NW - 1) / NW, VS1 = (RV::NJ1 + NW - 1) / NW;
 
-    extern __shared__ __attribute__((aligned(16))) char lds[];      // the staged tiles, the next work item, (kDirect) the exchange area
+    extern __shared__ __attribute__((aligned(16))) char lds[];      // the staged tiles, the next work item, the exchange area, ...
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -133,10 +127,10 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // (Direct loads: the two wavefronts of a tile of 16 q heads share the dot products as well - the one with the even
         // k-steps, the other with the odd ones, KQ = KS / 2 each - and exchange their halves through LDS: half the reads of
         // the staged K rows, half the Q^T registers.)
-        constexpr int KQ = kDirect ? KS / CS : KS;                  // k-steps of this wavefront: ks = kq_step * i + kq_first
-        constexpr int kq_step = kDirect ? CS : 1;
-        const int kq_first = kDirect ? whalf : 0;
-        static_assert(!kDirect || (KS % CS == 0 && CS == 2), "the k-steps split by parity");
+        constexpr int KQ = KS / CS;                                 // k-steps of this wavefront: ks = kq_step * i + kq_first
+        constexpr int kq_step = CS;
+        const int kq_first = whalf;
+        static_assert(KS % CS == 0 && CS == 2, "the k-steps split by parity");
         uint4 qreg[KQ];
 #pragma unroll
         for (int i = 0; i < KQ; ++i) qreg[i] = make_uint4(0, 0, 0, 0);
@@ -148,7 +142,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 for (int i = 0; i < KQ; ++i) qreg[i] = *reinterpret_cast<const uint4*>(qp + 32 * kq_step * i);
             }
         };
-        if (!kDirect) load_q();                 // (direct loads: requested behind the first rows, see the tile loop)
         const ConstI32 tbl = as_const(p.block_table + (int64_t)b * p.tbl_sb);
         const int pmask = p.page_size - 1;
         const int kv_len = min(as_const(p.kv_lens)[b], p.max_tokens);
@@ -187,14 +180,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         const char* vplane = reinterpret_cast<const char*>(p.v) + ((int64_t)kvh * p.v_sh) * ES;
         const uint32_t ksp_bytes = (uint32_t)(p.k_sp * ES), vsp_bytes = (uint32_t)(p.v_sp * ES);
         const uint32_t kst_bytes = (uint32_t)(p.k_st * ES), vst_bytes = (uint32_t)(p.v_st * ES);
-        // rows that the other workgroups of the group read as well stay in the XCD's L2 (plain loads); rows that are
-        // read once come with the non-temporal hint
-        auto load16 = [&](const char* ptr) { return REUSE ? *reinterpret_cast<const uint4*>(ptr) : load_stream16(ptr); };
-
-        struct Tile {                                               // this wavefront's share of a tile, as loaded
-            uint32_t k[KS0 + KS1][4];
-            uint32_t v[VS0 + VS1][4];
-        };
         // Load instruction j of a segment covers rows j * RPL .. + RPL - 1 (a lane: row j * RPL + lane / LPR, 16 bytes
         // from byte seg + (lane % LPR) * 16 of the cache row); wavefront w issues the instructions j = w, w + 4, ...
         // This lane's place within the rows of a load instruction, as a byte offset from the first row (one value per
@@ -228,11 +213,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             const uint32_t pg = (uint32_t)(PM == PM_TILE ? pg_id : __shfl(pg_id, n - tok0, 64));
             return plane + ((uint64_t)pg * sp_bytes + (uint64_t)(slot * st_bytes)) + lane_byte;
         };
-        auto load_rows = [&](auto clamp_tag, int tok0, int32_t pg_id, int first_row, int lane_row, uint32_t lane_off,
-                             uint32_t lane_byte, const char* plane, uint32_t sp_bytes, uint32_t st_bytes) {
-            return load16(row_ptr(clamp_tag, tok0, pg_id, first_row, lane_row, lane_off, lane_byte, plane, sp_bytes, st_bytes));
-        };
-        // ---- direct loads (kDirect): 16 bytes per lane from memory to LDS byte (dst + 16 lane), dst wave-uniform.  The
+        // ---- direct loads: 16 bytes per lane from memory to LDS byte (dst + 16 lane), dst wave-uniform.  The
         // compiler does not see these loads (it would wait for ALL loads under way in front of every LDS read that follows
         // one): the tile loop places its own waits, see there. ----
         auto load_to_lds16 = [&](const char* ptr, uint32_t dst) {
@@ -269,8 +250,8 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 load_to_lds16(row_ptr(clamp_tag, tok0, pg_id, j, 0, byte, byte, vplane, vsp_bytes, vst_bytes), dst + kTile * RBK + j * 1024);
             }
         };
-        // ---- e4m3 rows through raw tiles (kRaw).  The load instructions and their lanes are those of the register path
-        // (issue): instruction j of a segment covers rows j RPL .., 16 bytes per lane; it fills 1 KB of the raw tile, first K
+        // ---- e4m3 rows through raw tiles (kRaw): load instruction j of a segment covers rows j RPL .. (a lane: row j RPL + lane /
+        // LPR, 16 bytes from byte (lane % LPR) 16 of the segment); it fills 1 KB of the raw tile, first K
         // segments, second K segment, V rows.  convert_raw reads back exactly the bytes this wavefront requested. ----
         // Two raw tiles of first K segments and V rows, each wavefront reading back only what it requested itself; the
         // second K segment, one instruction that every wavefront issues and converts alike (so that all issue the same
@@ -369,13 +350,33 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // last token) into one of eight slots behind the exchange area, and the requests for the rows read them from there,
         // by then long landed (see the tile loop).  All wavefronts write the same numbers to the same place.
         constexpr int kPageSlots = 8;
-        const uint32_t pg_lds = (uint32_t)(kStaged * kTileBytes + 16 + 2 * NW * 1024);    // offset of the slots from lds[0]
+        const uint32_t pg_lds = (uint32_t)(kStaged * kTileBytes + 16 + 2 * NW * 1024 + (kRaw ? 2 * (RK::NJ0 + RV::NJ0) * 1024 + 4 * 1024 : 0));    // offset of the slots from lds[0] (behind the raw tiles)
         auto issue_pages = [&](int t) {
             const int n = min(c_start + t * kTile + (lane & 15), c_end - 1);
             const int idx = p.page_shift < 0 ? n / p.page_size : n >> p.page_shift;
             const int32_t* ptr = p.block_table + (int64_t)b * p.tbl_sb + idx;
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(ptr), "s"(lds0 + pg_lds + (uint32_t)(t & (kPageSlots - 1)) * 256)
                          : "memory");
+        };
+        // e4m3 rows with page numbers per row: every lane reads the number of its row from the slot.
+        auto issue_raw_rows = [&](int t) {
+            const int tok0 = c_start + t * kTile;
+            const int32_t* pages = reinterpret_cast<const int32_t*>(lds + pg_lds + (t & (kPageSlots - 1)) * 256);
+            const uint32_t dst = lds0 + raw_lds + (uint32_t)(t & 1) * kRawTile;
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            ln &= 63;
+            auto place = [&](int n) { return p.page_shift < 0 ? (uint32_t)(n % p.page_size) : (uint32_t)(n & pmask); };
+            static_assert(!kRaw || (KS0 == 1 && KS1 == 1 && VS0 == 1), "one instruction per segment and wavefront");
+            const int j0 = slot_instr(0, RK::NJ0), j1 = slot_instr(0, RK::NJ1), jv = slot_instr(0, RV::NJ0);
+            const int row0 = j0 * RK::RPL0 + ln / RK::LPR0, row1 = j1 * RK::RPL1 + ln / RK::LPR1, rowv = jv * RV::RPL0 + ln / RV::LPR0;
+            const uint32_t pg0 = (uint32_t)pages[row0], pg1 = (uint32_t)pages[row1], pgv = (uint32_t)pages[rowv];
+            const uint32_t pl0 = place(min(tok0 + row0, c_end - 1)), pl1 = place(min(tok0 + row1, c_end - 1)),
+                           plv = place(min(tok0 + rowv, c_end - 1));
+            load_to_lds16(kplane + ((uint64_t)pg0 * ksp_bytes + (uint64_t)(pl0 * kst_bytes)) + (ln % RK::LPR0) * 16, dst + j0 * 1024);
+            load_to_lds16(kplane + ((uint64_t)pg1 * ksp_bytes + (uint64_t)(pl1 * kst_bytes)) + (RK::D0 * ES + (ln % RK::LPR1) * 16),
+                          lds0 + raw1_lds + (uint32_t)(t & 3) * (RK::NJ1 * 1024) + j1 * 1024);
+            load_to_lds16(vplane + ((uint64_t)pgv * vsp_bytes + (uint64_t)(plv * vst_bytes)) + (ln % RV::LPR0) * 16, dst + (RK::NJ0 + jv) * 1024);
         };
         // Tile t with page numbers per row.  A first-segment instruction covers ONE row: its page number, read from the slot
         // by every lane alike, its place in the page and with them its address are wave-uniform.  The instruction of the
@@ -421,110 +422,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                 load_to_lds16(vplane + v_base[s] + (uint32_t)((ln ^ ((j & 3) << 1)) << 4), dst + kTile * RBK + j * 1024);
             }
         };
-        auto issue = [&](auto clamp_tag, int t, int32_t pg_id, Tile& rg) {
-            const int tok0 = c_start + t * kTile;
-            int ln = lane;                                  // (as in stage below)
-            asm volatile("" : "+v"(ln));
-            ln &= 63;                                       // (known to the compiler again: a row of 64 lanes is one row)
-#pragma unroll
-            for (int s = 0; s < KS0; ++s) {
-                const int j = slot_instr(s, RK::NJ0);
-                    put(rg.k[s], load_rows(clamp_tag, tok0, pg_id, j * RK::RPL0, ln / RK::LPR0, k_lane0, (ln % RK::LPR0) * 16,
-                                           kplane, ksp_bytes, kst_bytes));
-            }
-#pragma unroll
-            for (int s = 0; s < KS1; ++s) {
-                const int j = slot_instr(s, RK::NJ1);
-                    put(rg.k[KS0 + s], load_rows(clamp_tag, tok0, pg_id, j * RK::RPL1, ln / RK::LPR1, k_lane1,
-                                                 RK::D0 * ES + (ln % RK::LPR1) * 16, kplane, ksp_bytes, kst_bytes));
-            }
-#pragma unroll
-            for (int s = 0; s < VS0; ++s) {
-                const int j = slot_instr(s, RV::NJ0);
-                    put(rg.v[s], load_rows(clamp_tag, tok0, pg_id, j * RV::RPL0, ln / RV::LPR0, v_lane0, (ln % RV::LPR0) * 16,
-                                           vplane, vsp_bytes, vst_bytes));
-            }
-#pragma unroll
-            for (int s = 0; s < VS1; ++s) {
-                const int j = slot_instr(s, RV::NJ1);
-                    put(rg.v[VS0 + s], load_rows(clamp_tag, tok0, pg_id, j * RV::RPL1, ln / RV::LPR1, v_lane1,
-                                                 RV::D0 * ES + (ln % RV::LPR1) * 16, vplane, vsp_bytes, vst_bytes));
-            }
-        };
-        // registers -> the shared staged tile (swizzled like the private tiles of the other kernels)
-        auto stage = [&](const Tile& rg, char* buf) {
-            char* lk = buf;
-            char* lv = buf + kTile * RBK;
-            // (the lane number through an empty asm: the per-lane parts of the store addresses are then computed here, a
-            // few operations each, instead of being kept in registers - or spilled, and a spill reload waits for every
-            // load under way - across the tile loop)
-            int ln = lane;
-            asm volatile("" : "+v"(ln));
-            ln &= 63;                                       // (known to the compiler again: a row of 64 lanes is one row)
-            // one register quadruple to its place in a staged row: 16 bytes of a 16-bit cache are one chunk; 16 one-byte
-            // values become two chunks of 16-bit values
-            auto store_k = [&](const uint32_t (&r)[4], int row, int piece) {
-                if constexpr (!FP8) {
-                    *reinterpret_cast<uint4*>(lk + k_off<RBK>(row, piece)) = get(r);
-                } else {
-                    uint32_t o[8];
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        if (fold) {
-                            o[2 * w] = P2::from_fp8(r[w], false, kconv);
-                            o[2 * w + 1] = P2::from_fp8(r[w], true, kconv);
-                        } else {
-                            const f32x2_t k01 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], false);
-                            const f32x2_t k23 = __builtin_amdgcn_cvt_pk_f32_fp8(r[w], true);
-                            o[2 * w] = P2::pack(k01.x * kscale, k01.y * kscale);
-                            o[2 * w + 1] = P2::pack(k23.x * kscale, k23.y * kscale);
-                        }
-                    }
-#pragma unroll
-                    for (int half = 0; half < 2; ++half)
-                        *reinterpret_cast<uint4*>(lk + k_off<RBK>(row, 2 * piece + half)) =
-                            make_uint4(o[4 * half], o[4 * half + 1], o[4 * half + 2], o[4 * half + 3]);
-                }
-            };
-            auto store_v = [&](const uint32_t (&r)[4], int row, int piece) {
-                if constexpr (!FP8) {
-                    *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, piece)) = get(r);
-                } else {
-                    uint32_t o[8];
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        o[2 * w] = P2::from_fp8(r[w], false);
-                        o[2 * w + 1] = P2::from_fp8(r[w], true);
-                    }
-#pragma unroll
-                    for (int half = 0; half < 2; ++half)
-                        *reinterpret_cast<uint4*>(lv + v_off<RBV>(row, 2 * piece + half)) =
-                            make_uint4(o[4 * half], o[4 * half + 1], o[4 * half + 2], o[4 * half + 3]);
-                }
-            };
-            // (piece: the lane's 16 bytes within the cache row, counted in 16-byte pieces)
-#pragma unroll
-            for (int s = 0; s < KS0; ++s) {
-                const int j = slot_instr(s, RK::NJ0);
-                store_k(rg.k[s], j * RK::RPL0 + ln / RK::LPR0, ln % RK::LPR0);
-            }
-#pragma unroll
-            for (int s = 0; s < KS1; ++s) {
-                const int j = slot_instr(s, RK::NJ1);
-                store_k(rg.k[KS0 + s], j * RK::RPL1 + ln / RK::LPR1, RK::D0 * ES / 16 + ln % RK::LPR1);
-            }
-#pragma unroll
-            for (int s = 0; s < VS0; ++s) {
-                const int j = slot_instr(s, RV::NJ0);
-                store_v(rg.v[s], j * RV::RPL0 + ln / RV::LPR0, ln % RV::LPR0);
-            }
-#pragma unroll
-            for (int s = 0; s < VS1; ++s) {
-                const int j = slot_instr(s, RV::NJ1);
-                store_v(rg.v[VS0 + s], j * RV::RPL1 + ln / RV::LPR1, RV::D0 * ES / 16 + ln % RV::LPR1);
-            }
-        };
-
         // Online softmax against a REFERENCE maximum that moves rarely.  The output tile lives in the accumulation
         // registers, which only the matrix cores reach directly; a rescale by exp2(old max - new max) goes through the
         // vector ALU, i.e. through copies of all 128 registers, and with the rescale inside the tile loop the compiler
@@ -564,47 +461,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             //   K operand of k-step ks: row c, chunk 4 ks + a  ->  chunk ^ (c & 7) = 8 (ks >> 1) + ((4 (ks & 1) + a) ^ (c & 7))
             //   V operand of block db (transposed read): row 4 a + (c >> 2), chunk 2 db + ((c & 3) >> 1)
             //                                            ->  2 (4 (db >> 2) + ((db & 3) ^ (row & 3))) + ((c & 3) >> 1)
-        auto qk_tile = [&](const char* buf) {
-            if constexpr (kDirect) {
-                return f32x4_t{0.f, 0.f, 0.f, 0.f};     // (not used: qk_half)
-            } else {
-            const char* lk = buf + c * kK0Row;
-            const char* k_at[2] = {lk + (((0 + a) ^ (c & 7)) << 4), lk + (((4 + a) ^ (c & 7)) << 4)};
-            // (k-steps of the second K segment: from row c's second segment on, which in the direct-load layout lies
-            // elsewhere than behind its first)
-            constexpr int KSEG0 = RK::D0 / 32;
-            const int k1_delta = kK1Base + c * (kK1Row - kK0Row) - KSEG0 / 2 * 128;
-            // ---- S^T[token][head] = K Q^T: QG accumulation chains; the K operands of the next QG k-steps are requested
-            // from LDS before the MFMA of the current ones (and no further ahead: every operand held in registers is
-            // one the output tile and the loads under way cannot have) ----
-            constexpr int QG = 6, NQG = KS / QG;
-            static_assert(KS % QG == 0, "k-steps in whole groups");
-            f32x4_t s3[QG];
-#pragma unroll
-            for (int i = 0; i < QG; ++i) s3[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            uint4 ka[2][QG];
-            auto read_qk = [&](int g, int to) {
-#pragma unroll
-                for (int i = 0; i < QG; ++i) {
-                    const int ks = g * QG + i;
-                    if (kDirect && ks >= KSEG0) ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + k1_delta + (ks >> 1) * 128);
-                    else ka[to][i] = *reinterpret_cast<const uint4*>(k_at[ks & 1] + (ks >> 1) * 128);
-                }
-            };
-            read_qk(0, 0);
-#pragma unroll
-            for (int g = 0; g < NQG; ++g) {
-                if (g + 1 < NQG) read_qk(g + 1, (g + 1) & 1);
-#pragma unroll
-                for (int i = 0; i < QG; ++i) s3[i] = M::qk(ka[g & 1][i], qreg[g * QG + i], s3[i]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            f32x4_t s = s3[0];
-#pragma unroll
-            for (int i = 1; i < QG; ++i) s += s3[i];
-            return s;
-            }
-        };
         // Direct loads: this wavefront's half of the dot products, k-steps kq_first, kq_first + 2, ...: the operands of its
         // parity class are 128 bytes apart from ONE base address (the last k-step lies in the second K segment).
         auto qk_half = [&](const char* buf) {
@@ -682,7 +538,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             }
             return true;
         };
-        auto try_compute = [&](int t, const char* buf, auto masked_tag) { return softmax_pv(t, buf, qk_tile(buf), masked_tag); };
 
         // ---- the tiles of the piece: the loads of tiles t + 1 and t + 2 are under way while all wavefronts work on tile t
         // (two register tiles by the parity of t; the memory system's latency is longer than the arithmetic of one tile).
@@ -690,7 +545,7 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
         // in order, so waiting for a number then never waits for rows requested after it.
         // (A wavefront that leaves the inner loop to move its reference does so after the tile's barrier and comes back for
         // the next tile: every wavefront passes exactly one barrier per tile.) ----
-        if constexpr (kDirect) {
+        {
             // Direct loads, four staged tiles (tile t in buffer t % 4), and the arithmetic of two tiles in one step: the dot
             // products of tile t + 1 next to the softmax and the PV product of tile t, which do not depend on each other - the
             // matrix cores work on the one while the vector ALU and the LDS round trips of the other are under way (with one
@@ -706,8 +561,13 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             auto issue_tile = [&](int t, int32_t pg_id) {
                 const uint32_t dst = lds0 + (uint32_t)(t % kStaged) * kTileBytes;
                 if constexpr (kRaw) {
-                    if (t < n_full) issue_raw(BoolTag<false>(), t, pg_id);
-                    else if (t < n_tiles) issue_raw(BoolTag<true>(), t, pg_id);
+                    if (PM == PM_ROW) {
+                        if (t < n_tiles) issue_raw_rows(t);
+                    } else if (t < n_full) {
+                        issue_raw(BoolTag<false>(), t, pg_id);
+                    } else if (t < n_tiles) {
+                        issue_raw(BoolTag<true>(), t, pg_id);
+                    }
                 } else if (PM == PM_ROW) {
                     if (t < n_tiles) issue_direct_rows(t, dst);
                 } else if (t < n_full) {
@@ -722,18 +582,39 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
             // kRaw: one round of a tile's bytes - wait until this wavefront's share of tile u has landed in its raw tile (its
             // loads return in order: all but those of tile u + 1), convert it into the staged tile, request tile u + 2 into
             // the raw tile just read.
+            // (Page numbers per row: a round requests the bytes of tile u + 2 and then the page numbers of tile u + 4; what
+            // has to have landed at its top are the bytes of tile u and the page numbers of tile u + 2, requested two rounds
+            // ago in that order: everything but the loads of the round before.)
             auto advance_raw = [&](int u) {
-                if (u + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerTile) : "memory");
-                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                if (u < n_tiles) convert_raw(u, staged(u));
-                const int32_t pg_now = pg_hold;
-                pg_hold = page_id(u + 3);
-                issue_tile(u + 2, pg_now);
+                if (PM == PM_ROW) {
+                    if (u + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerTile + 1) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+                    if (u < n_tiles) convert_raw(u, staged(u));
+                    issue_tile(u + 2, 0);
+                    issue_pages(u + 4);
+                } else {
+                    if (u + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerTile) : "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    if (u < n_tiles) convert_raw(u, staged(u));
+                    const int32_t pg_now = pg_hold;
+                    pg_hold = page_id(u + 3);
+                    issue_tile(u + 2, pg_now);
+                }
             };
             if constexpr (kRaw) {
-                issue_tile(0, page_id(0));
-                issue_tile(1, page_id(1));
-                pg_hold = page_id(2);
+                if (PM == PM_ROW) {
+                    issue_pages(0);
+                    issue_pages(1);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    issue_tile(0, 0);
+                    issue_pages(2);
+                    issue_tile(1, 0);
+                    issue_pages(3);
+                } else {
+                    issue_tile(0, page_id(0));
+                    issue_tile(1, page_id(1));
+                    pg_hold = page_id(2);
+                }
                 advance_raw(0);
                 advance_raw(1);
             } else if (PM == PM_ROW) {
@@ -827,50 +708,6 @@ __global__ __launch_bounds__(64 * kSharedWaves) void splitkv_mfma_shared_kernel(
                     while (!softmax_pv(n_full, staged(n_full), s_cur, BoolTag<true>())) move_reference();
                 }
             }
-        } else {
-            Tile rg_even, rg_odd;
-            const int n_full = (c_end - c_start) / kTile;          // tiles without rows past the end
-            auto issue_tile = [&](int t, int32_t pg_id, Tile& rg) {
-                if (t < n_full) issue(BoolTag<false>(), t, pg_id, rg);
-                else if (t < n_tiles) issue(BoolTag<true>(), t, pg_id, rg);
-            };
-            int32_t pg_even = page_id(0), pg_odd = page_id(1);
-            issue_tile(0, pg_even, rg_even);
-            pg_even = page_id(2);
-            issue_tile(1, pg_odd, rg_odd);
-            pg_odd = page_id(3);
-            // tile t up to its barrier: stage it, request the rows of tile t + 2 into the registers it came from
-            auto stage_and_issue = [&](int t, Tile& rg, int32_t& pg) {
-                stage(rg, lds + (t & 1) * kTileBytes);              // waits for this wavefront's loads of tile t
-                issue_tile(t + 2, pg, rg);
-                pg = page_id(t + 4);
-                // tile t is staged; tile t - 1 has been read by everyone.  (The barrier waits for this wavefront's LDS
-                // operations only: __syncthreads() would also wait for the rows just requested from memory, i.e. for the
-                // very loads that are meant to be under way during the arithmetic.)
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            };
-            int t = 0;
-            for (;;) {
-                bool gave_up = false;
-                for (; t < n_full; ++t) {
-                    if (t & 1) stage_and_issue(t, rg_odd, pg_odd);
-                    else stage_and_issue(t, rg_even, pg_even);
-                    if (active && !try_compute(t, lds + (t & 1) * kTileBytes, BoolTag<false>())) {
-                        gave_up = true;
-                        break;
-                    }
-                }
-                if (!gave_up) break;
-                do move_reference(); while (!try_compute(t, lds + (t & 1) * kTileBytes, BoolTag<false>()));
-                ++t;
-            }
-            if (n_full < n_tiles) {                                 // the partial last tile
-                if (n_full & 1) stage_and_issue(n_full, rg_odd, pg_odd);
-                else stage_and_issue(n_full, rg_even, pg_even);
-                if (active) {
-                    while (!try_compute(n_full, lds + (n_full & 1) * kTileBytes, BoolTag<true>())) move_reference();
-                }
-            }
         }
         if (!active) return;
 
@@ -913,11 +750,10 @@ int launch_shared(const SplitParams& p_in, hipStream_t stream) {
     SplitParams p = p_in;
     p.head_tiles = (p.group + kSharedTileHeads - 1) / kSharedTileHeads;
     p.hg_blocks = p.hkv;
-    // staged tiles, the next work item, and (direct loads) the exchange area of the half dot products: see kDirect
+    // staged tiles, the next work item, the exchange area of the half dot products, ...
     const int pm = (p.page_shift >= 0 && p.page_size % kTile == 0) ? PM_TILE : PM_ROW;
     const size_t lds_bytes = !FP8 ? 4 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 8 * 256      // (+ page numbers)
-                           : pm == PM_TILE ? 3 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 2 * 16384 + 4 * 1024   // (+ raw tiles)
-                                           : 2 * (size_t)kTileBytes + 16;
+                           : 3 * (size_t)kTileBytes + 16 + 2 * kSharedWaves * 1024 + 2 * 16384 + 4 * 1024 + 8 * 256;   // (+ raw tiles, page numbers)
     p.total_items = (int32_t)((int64_t)p.batch * p.num_splits * p.hg_blocks * p.head_tiles);
     // (the work queue: as many workgroups as are resident at once - one per compute unit at this size - and never more
     // than there are pieces: every workgroup of the queue has to take one, or it would not be counted among the
